@@ -1,0 +1,200 @@
+/*
+ * sbnet_amd.h -- C ABI of libsbnet_amd.so: the three Sparse Blocks Network custom ops
+ * (reduce_mask, sparse_gather, sparse_scatter / sparse_scatter_var) as hand-written HIP kernels
+ * for gfx950 (MI355X).
+ *
+ * The entry points replace the reference's TensorFlow op kernels and the functors below them
+ * (paths relative to the reference checkout, sbnet_tensorflow/sbnet_ops/).  Two levels exist,
+ * as in the reference:
+ *
+ *   op level       what OpKernel::Compute does: parameter validation, the host-visible count,
+ *                  the zero-count fix-up, copy-before-scatter.   Names: sbnet_<op>.
+ *   functor level  what Functor<GPUDevice,float>::operator() does: launch only, reference
+ *                  argument order.                               Names: sbnet_<op>_functor.
+ *
+ * Conventions
+ *   - Only float32 tensors, NHWC, C-contiguous.  Block indices are int16 triples (n, bh, bw)
+ *     (reduce_mask.cc:109, sparse_gather.cc:53).
+ *   - The caller owns every buffer.  Pointers are device pointers unless a parameter says "host".
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  All work is
+ *     enqueued on it; only sbnet_reduce_mask with a host count pointer waits for it.
+ *   - The dynamic_b* parameters are host int32 arrays with an explicit length so that the
+ *     reference's "should be one-dimensional with shape[0] == 2" check can be mirrored.
+ *   - Every function returns an sbnet_status.  No function ever calls exit(); the reference
+ *     prints and exits on a device error (op_utils.h:27-35), this library returns SBNET_EHIP.
+ *   - Re-entrant: no global mutable state apart from a thread-local last-error slot.
+ */
+#ifndef SBNET_AMD_H
+#define SBNET_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum sbnet_status {
+    SBNET_OK = 0,
+    /* dynamic_b<count,size,stride,offset> not length 2
+       (reduce_mask.cc:132-138, sparse_gather.cc:169-175, 307-313). */
+    SBNET_EINVAL_PARAM_SHAPE = 1,
+    /* x / ybase not rank 4 (sparse_gather.cc:164, 327). */
+    SBNET_EINVAL_RANK = 2,
+    /* add && !atomic with bstride < bsize (sparse_gather.cc:322-326). */
+    SBNET_EINVAL_OVERLAP = 3,
+    /* Anything the reference does not check but that would make a kernel read or write out of
+       bounds: NULL pointers, non-positive sizes, dimensions beyond the int16 index range,
+       a workspace that is too small, y aliasing ybase in the copying scatter. */
+    SBNET_EINVAL_ARG = 4,
+    /* A HIP runtime call failed; sbnet_last_hip_error() has the hipError_t. */
+    SBNET_EHIP = 5
+} sbnet_status;
+
+/* Human-readable text for a status; the InvalidArgument texts are the reference's. */
+const char* sbnet_status_string(int status);
+/* hipError_t of the last SBNET_EHIP on the calling thread (0 if none). */
+int sbnet_last_hip_error(void);
+const char* sbnet_version(void);
+
+/* ------------------------------------------------------------------------------------------
+ * reduce_mask
+ * ---------------------------------------------------------------------------------------- */
+
+/* Rows of active_block_indices the caller must allocate: N * bcount[0] * bcount[1]
+   (reduce_mask.cc:161).  Returns -1 on bad arguments. */
+int64_t sbnet_reduce_mask_max_indices(int N, const int32_t* bcount, int bcount_len);
+
+/* Bytes of device scratch sbnet_reduce_mask / _functor need for this problem size. */
+size_t sbnet_reduce_mask_workspace_bytes(int N, const int32_t* bcount, int bcount_len);
+
+/*
+ * Op level: replaces ReduceMaskOp<GPUDevice,float>::Compute (reduce_mask.cc:123-221).
+ *
+ *   mask                  device fp32 [N,H,W,1]
+ *   bcount/bsize/bstride/boffset   host int32[2] each (len must be 2)
+ *   tol, avgpool          op attributes (reduce_mask.cc:102-103).  max mode: active if any
+ *                         in-range pixel > tol.  avg mode: active if sum(in-range)/(bsize[0]*
+ *                         bsize[1]) > tol, with the sum taken in the CPU functor's row-major
+ *                         order (reduce_mask.cc:78-88), so results are identical to the
+ *                         reference's CPU path for any mask, not only binary ones.
+ *   active_block_indices  device int16 [max_indices, 3].  Unlike the reference's GPU kernel
+ *                         (arbitrary order, reduce_mask.cu.h:141-154) rows are written in the
+ *                         CPU functor's lexicographic (n, bh, bw) order.  Rows past the count
+ *                         are left untouched.
+ *   bin_counts_host       host int32[1] or NULL.  Non-NULL keeps the reference's HostMemory
+ *                         contract (reduce_mask.cc:198-220): the count is copied back and the
+ *                         call returns after the stream has drained.  NULL: nothing is copied,
+ *                         the call is asynchronous.
+ *   bin_counts_device     device int32[1] or NULL; receives the same count.  At least one of
+ *                         the two count pointers must be non-NULL.
+ *   A mask with no active block reports count 1 and writes the triple (0,0,0)
+ *   (reduce_mask.cc:206-218); the fix-up happens on the device, without a host round trip.
+ *   workspace             device scratch of sbnet_reduce_mask_workspace_bytes() bytes, 16-byte
+ *                         aligned, or NULL to let the call allocate and free its own
+ *                         (slower, and it synchronises the stream).
+ */
+int sbnet_reduce_mask(const float* mask, int N, int H, int W,
+                      const int32_t* bcount, int bcount_len,
+                      const int32_t* bsize, int bsize_len,
+                      const int32_t* bstride, int bstride_len,
+                      const int32_t* boffset, int boffset_len,
+                      float tol, int avgpool,
+                      int16_t* active_block_indices,
+                      int32_t* bin_counts_host, int32_t* bin_counts_device,
+                      void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Functor level: replaces ReduceMaskFunctor<GPUDevice,float>::operator()
+ * (reduce_mask.h:23-44, reduce_mask.cu:39-89).  Same argument order; numBins must be 1 as the
+ * reference asserts (reduce_mask.cc:69), binSize is ignored.  binCounts is a device int32[1]
+ * and receives the raw count (0 is possible: the fix-up belongs to the op level).
+ */
+int sbnet_reduce_mask_functor(const float* mask, int N, int H, int W, float threshold,
+                              int bOffsH0, int bOffsW0, int bSzH, int bSzW, int bStrH, int bStrW,
+                              int bCntH, int bCntW, unsigned int numBins, unsigned int binSize,
+                              int16_t* activeBlockIndices, int32_t* binCounts, int avgPool,
+                              void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * sparse_gather
+ * ---------------------------------------------------------------------------------------- */
+
+/*
+ * Op level: replaces SparseGatherOp<GPUDevice,float>::Compute (sparse_gather.cc:160-218).
+ *
+ *   x, x_dims, x_rank     device fp32 NHWC and its shape; rank must be 4
+ *   num_active            bin_counts[0], which the reference reads on the host
+ *                         (sparse_gather.cc:190-192)
+ *   active_block_indices  device int16 [>= num_active, 3]
+ *   transpose             0: y is [num_active, bsize[0], bsize[1], C]
+ *                         1: y is [num_active, C, bsize[0], bsize[1]]  (sparse_gather.cc:197-204)
+ *   y                     device fp32, caller-allocated with that shape
+ *   Pixels outside the image read as 0 (sparse_gather.cc:80-82).
+ */
+int sbnet_sparse_gather(const float* x, const int64_t* x_dims, int x_rank,
+                        int32_t num_active, const int16_t* active_block_indices,
+                        const int32_t* bsize, int bsize_len,
+                        const int32_t* bstride, int bstride_len,
+                        const int32_t* boffset, int boffset_len,
+                        int transpose, float* y, void* stream);
+
+/* Functor level: replaces SparseGatherFunctor<GPUDevice,float>::operator()
+   (sparse_gather.h:23-42, sparse_gather.cu:62-154). */
+int sbnet_sparse_gather_functor(const float* x, int N, int H, int W, int C, float* y,
+                                int bOffsH0, int bOffsW0, int bSzH, int bSzW, int bStrH, int bStrW,
+                                int numActive, const int16_t* activeBlockIndices, int transpose,
+                                void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * sparse_scatter / sparse_scatter_var
+ * ---------------------------------------------------------------------------------------- */
+
+/*
+ * Op level: replaces SparseScatterOp<GPUDevice,float,false>::Compute (sparse_gather.cc:286-357,
+ * registered as "SparseScatter", sparse_gather.cc:256-268): y = copy(ybase), then the blocks of
+ * x are written (add=0), added (add=1) or atomically added (add=1, atomic=1) on top of y.
+ * Unlike the reference (sparse_gather.cu:268-276) the copy does not synchronise the stream.
+ *
+ *   x           device fp32 block stack: [num_active, bsize[0], bsize[1], C], or
+ *               [num_active, C, bsize[0], bsize[1]] when transpose=1 (sparse_gather.cc:117-120)
+ *   ybase       device fp32 [N,H,W,C]; ybase_dims/ybase_rank give its shape, rank must be 4
+ *   y           device fp32, same shape, must not overlap ybase
+ *   Pixels of a block that fall outside the image are dropped (sparse_gather.cc:121).
+ *   add=1, atomic=0 requires bstride >= bsize on both axes (sparse_gather.cc:322-326).
+ *   add=0 with overlapping blocks: as in the reference's GPU path, which block wins on an
+ *   overlapped pixel is unspecified unless the overlapping values are equal.
+ */
+int sbnet_sparse_scatter(const float* x, int32_t num_active, const int16_t* active_block_indices,
+                         const float* ybase, const int64_t* ybase_dims, int ybase_rank,
+                         const int32_t* bsize, int bsize_len,
+                         const int32_t* bstride, int bstride_len,
+                         const int32_t* boffset, int boffset_len,
+                         int add, int atomic, int transpose, float* y, void* stream);
+
+/* Op level, in place: replaces SparseScatterOp<GPUDevice,float,true>::Compute ("SparseScatterVar",
+   sparse_gather.cc:242-254, 335-337).  ybase is modified and is the result. */
+int sbnet_sparse_scatter_var(const float* x, int32_t num_active,
+                             const int16_t* active_block_indices,
+                             float* ybase, const int64_t* ybase_dims, int ybase_rank,
+                             const int32_t* bsize, int bsize_len,
+                             const int32_t* bstride, int bstride_len,
+                             const int32_t* boffset, int boffset_len,
+                             int add, int atomic, int transpose, void* stream);
+
+/* Functor level: replaces SparseScatterFunctor<GPUDevice,float>::operator()
+   (sparse_gather.h:45-66, sparse_gather.cu:158-266).  Scatters into y in place, no validation
+   of the add/atomic/overlap combination. */
+int sbnet_sparse_scatter_functor(const float* x, int N, int H, int W, int C, float* y,
+                                 int bOffsH0, int bOffsW0, int bSzH, int bSzW, int bStrH,
+                                 int bStrW, int numActive, const int16_t* activeBlockIndices,
+                                 int add, int transpose, int atomic, void* stream);
+
+/* Replaces CopyTensorFunctor<GPUDevice,float>::operator() (sparse_gather.h:69-76,
+   sparse_gather.cu:268-276) without its stream synchronisation.  count is in floats. */
+int sbnet_copy_tensor(float* dst, const float* src, size_t count, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SBNET_AMD_H */

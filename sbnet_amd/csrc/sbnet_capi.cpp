@@ -1,0 +1,275 @@
+// C ABI of libsbnet_amd.so (declared in include/sbnet_amd.h): argument validation that mirrors
+// the reference ops' OP_REQUIRES checks, then the kernel launches of sbnet_kernels.hip.
+//
+// Reference behaviour reproduced here (sbnet_tensorflow/sbnet_ops/):
+//   reduce_mask.cc:132-138, 141-220   parameter shape check, host-visible count, zero-count fix-up
+//   sparse_gather.cc:164-175, 190-207 rank / parameter checks, count taken from the host
+//   sparse_gather.cc:307-346          parameter checks, add/atomic/overlap rule, rank check,
+//                                     in place (Var) versus copy-then-scatter
+#include "../../include/sbnet_amd.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include "sbnet_launch.h"
+
+namespace {
+
+thread_local int g_lastHipError = 0;
+
+int hip_fail(hipError_t e)
+{
+    g_lastHipError = (int)e;
+    return SBNET_EHIP;
+}
+
+#define SBNET_HIP(call)                                  \
+    do {                                                 \
+        hipError_t e_ = (call);                          \
+        if (e_ != hipSuccess) return hip_fail(e_);       \
+    } while (0)
+
+bool pair_ok(const int32_t* p, int len) { return p != nullptr && len == 2; }
+
+// Limits the reference leaves unchecked.  Indices are int16 triples, so n, bh and bw must fit.
+bool geom_ok(int N, int H, int W, int C, const int32_t* bsize, const int32_t* bstride)
+{
+    return N > 0 && H > 0 && W > 0 && C > 0 && bsize[0] > 0 && bsize[1] > 0 && bstride[0] > 0 &&
+           bstride[1] > 0 && (int64_t)N * H * W * C < (1ll << 40);
+}
+
+sbnet::Geom make_geom(int N, int H, int W, int C, const int32_t* bsize, const int32_t* bstride,
+                      const int32_t* boffset)
+{
+    sbnet::Geom g;
+    g.N = N; g.H = H; g.W = W; g.C = C;
+    g.R = bsize[0]; g.S = bsize[1];
+    g.U = bstride[0]; g.V = bstride[1];
+    g.oh = boffset[0]; g.ow = boffset[1];
+    return g;
+}
+
+bool dims_fit_int(const int64_t* d)
+{
+    for (int i = 0; i < 4; ++i)
+        if (d[i] < 0 || d[i] > 0x7fffffffll) return false;
+    return true;
+}
+
+int reduce_mask_impl(const float* mask, int N, int H, int W, const int32_t* bcount,
+                     const int32_t* bsize, const int32_t* bstride, const int32_t* boffset, float tol,
+                     int avgpool, bool fixup, int16_t* idx, int32_t* countHost, int32_t* countDev,
+                     void* workspace, size_t workspaceBytes, hipStream_t stream)
+{
+    if (!mask || !idx || (!countHost && !countDev)) return SBNET_EINVAL_ARG;
+    if (!geom_ok(N, H, W, 1, bsize, bstride)) return SBNET_EINVAL_ARG;
+    if (bcount[0] <= 0 || bcount[1] <= 0) return SBNET_EINVAL_ARG;
+    // (n, bh, bw) are stored as int16
+    if (N > 32768 || bcount[0] > 32768 || bcount[1] > 32768) return SBNET_EINVAL_ARG;
+    const int64_t T = (int64_t)N * bcount[0] * bcount[1];
+    if (T >= (1ll << 31)) return SBNET_EINVAL_ARG;
+    // block origins and ends must stay inside int arithmetic
+    const int64_t hEnd = (int64_t)boffset[0] + (int64_t)bstride[0] * (bcount[0] - 1) + bsize[0];
+    const int64_t wEnd = (int64_t)boffset[1] + (int64_t)bstride[1] * (bcount[1] - 1) + bsize[1];
+    if (hEnd > 0x7fffffffll || wEnd > 0x7fffffffll || (int64_t)bsize[0] * bsize[1] > 0x7fffffffll)
+        return SBNET_EINVAL_ARG;
+
+    const size_t need = sbnet::reduce_mask_workspace_bytes(T);
+    void* ws = workspace;
+    bool ownWs = false;
+    if (ws) {
+        if (workspaceBytes < need || (reinterpret_cast<uintptr_t>(ws) & 15)) return SBNET_EINVAL_ARG;
+    } else {
+        SBNET_HIP(hipMalloc(&ws, need));
+        ownWs = true;
+    }
+    const sbnet::Geom g = make_geom(N, H, W, 1, bsize, bstride, boffset);
+    hipError_t e = sbnet::launch_reduce_mask(mask, g, bcount[0], bcount[1], tol, avgpool != 0, fixup, idx,
+                                             countDev, ws, stream);
+    if (e == hipSuccess && countHost) {
+        // the count sits in countDev, or behind the flags and counts of the workspace
+        const int32_t* src = countDev;
+        if (!src) {
+            const size_t flagBytes = ((size_t)T + 15) & ~(size_t)15;
+            src = reinterpret_cast<const int32_t*>(static_cast<const uint8_t*>(ws) + flagBytes) + T;
+        }
+        e = hipMemcpyAsync(countHost, src, sizeof(int32_t), hipMemcpyDeviceToHost, stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(stream);
+    }
+    if (ownWs) {
+        hipError_t e2 = hipStreamSynchronize(stream);
+        hipError_t e3 = hipFree(ws);
+        if (e == hipSuccess) e = e2 != hipSuccess ? e2 : e3;
+    }
+    if (e != hipSuccess) return hip_fail(e);
+    return SBNET_OK;
+}
+
+int scatter_impl(const float* x, int32_t numActive, const int16_t* idx, float* out,
+                 const int64_t* dims, const int32_t* bsize, const int32_t* bstride,
+                 const int32_t* boffset, int add, int atomic, int transpose, hipStream_t stream)
+{
+    if (numActive < 0) return SBNET_EINVAL_ARG;
+    if (numActive > 0 && (!x || !idx)) return SBNET_EINVAL_ARG;
+    if (!out || !dims_fit_int(dims)) return SBNET_EINVAL_ARG;
+    if (!geom_ok((int)dims[0], (int)dims[1], (int)dims[2], (int)dims[3], bsize, bstride))
+        return SBNET_EINVAL_ARG;
+    const sbnet::Geom g = make_geom((int)dims[0], (int)dims[1], (int)dims[2], (int)dims[3], bsize, bstride, boffset);
+    const sbnet::ScatterMode mode =
+        !add ? sbnet::SCATTER_ASSIGN : (atomic ? sbnet::SCATTER_ATOMIC : sbnet::SCATTER_ADD);
+    SBNET_HIP(sbnet::launch_scatter(x, out, idx, numActive, g, transpose != 0, mode, stream));
+    return SBNET_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* sbnet_version(void) { return "sbnet_amd 0.1 (gfx950)"; }
+
+int sbnet_last_hip_error(void) { return g_lastHipError; }
+
+const char* sbnet_status_string(int status)
+{
+    switch (status) {
+    case SBNET_OK: return "OK";
+    case SBNET_EINVAL_PARAM_SHAPE:
+        return "InvalidArgument: dynamic_b<count, size, stride, offset> should be one-dimensional with shape[0] == 2.";
+    case SBNET_EINVAL_RANK: return "InvalidArgument: x / ybase must be rank 4";
+    case SBNET_EINVAL_OVERLAP:
+        return "InvalidArgument: Only non-overlapping blocks are supported with add=True, atomic=False";
+    case SBNET_EINVAL_ARG: return "InvalidArgument: null pointer, size out of range or workspace too small";
+    case SBNET_EHIP: return "HIP runtime error (see sbnet_last_hip_error)";
+    default: return "unknown sbnet status";
+    }
+}
+
+int64_t sbnet_reduce_mask_max_indices(int N, const int32_t* bcount, int bcount_len)
+{
+    if (!pair_ok(bcount, bcount_len) || N < 0 || bcount[0] < 0 || bcount[1] < 0) return -1;
+    return (int64_t)N * bcount[0] * bcount[1];
+}
+
+size_t sbnet_reduce_mask_workspace_bytes(int N, const int32_t* bcount, int bcount_len)
+{
+    const int64_t T = sbnet_reduce_mask_max_indices(N, bcount, bcount_len);
+    if (T < 0) return 0;
+    return sbnet::reduce_mask_workspace_bytes(T);
+}
+
+int sbnet_reduce_mask(const float* mask, int N, int H, int W, const int32_t* bcount, int bcount_len,
+                      const int32_t* bsize, int bsize_len, const int32_t* bstride, int bstride_len,
+                      const int32_t* boffset, int boffset_len, float tol, int avgpool,
+                      int16_t* active_block_indices, int32_t* bin_counts_host,
+                      int32_t* bin_counts_device, void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (!pair_ok(bcount, bcount_len) || !pair_ok(bsize, bsize_len) || !pair_ok(bstride, bstride_len) ||
+        !pair_ok(boffset, boffset_len))
+        return SBNET_EINVAL_PARAM_SHAPE;
+    return reduce_mask_impl(mask, N, H, W, bcount, bsize, bstride, boffset, tol, avgpool, true,
+                            active_block_indices, bin_counts_host, bin_counts_device, workspace,
+                            workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+int sbnet_reduce_mask_functor(const float* mask, int N, int H, int W, float threshold, int bOffsH0,
+                              int bOffsW0, int bSzH, int bSzW, int bStrH, int bStrW, int bCntH,
+                              int bCntW, unsigned int numBins, unsigned int binSize,
+                              int16_t* activeBlockIndices, int32_t* binCounts, int avgPool,
+                              void* workspace, size_t workspace_bytes, void* stream)
+{
+    (void)binSize;
+    if (numBins != 1 || !binCounts) return SBNET_EINVAL_ARG;  // reduce_mask.cc:69 asserts numBins == 1
+    const int32_t bcount[2] = {bCntH, bCntW}, bsize[2] = {bSzH, bSzW}, bstride[2] = {bStrH, bStrW},
+                  boffset[2] = {bOffsH0, bOffsW0};
+    return reduce_mask_impl(mask, N, H, W, bcount, bsize, bstride, boffset, threshold, avgPool, false,
+                            activeBlockIndices, nullptr, binCounts, workspace, workspace_bytes,
+                            static_cast<hipStream_t>(stream));
+}
+
+int sbnet_sparse_gather(const float* x, const int64_t* x_dims, int x_rank, int32_t num_active,
+                        const int16_t* active_block_indices, const int32_t* bsize, int bsize_len,
+                        const int32_t* bstride, int bstride_len, const int32_t* boffset,
+                        int boffset_len, int transpose, float* y, void* stream)
+{
+    if (x_rank != 4) return SBNET_EINVAL_RANK;  // sparse_gather.cc:164
+    if (!pair_ok(bsize, bsize_len) || !pair_ok(bstride, bstride_len) || !pair_ok(boffset, boffset_len))
+        return SBNET_EINVAL_PARAM_SHAPE;  // sparse_gather.cc:169-175
+    if (!x_dims || !dims_fit_int(x_dims)) return SBNET_EINVAL_ARG;
+    return sbnet_sparse_gather_functor(x, (int)x_dims[0], (int)x_dims[1], (int)x_dims[2], (int)x_dims[3], y,
+                                       boffset[0], boffset[1], bsize[0], bsize[1], bstride[0], bstride[1],
+                                       num_active, active_block_indices, transpose, stream);
+}
+
+int sbnet_sparse_gather_functor(const float* x, int N, int H, int W, int C, float* y, int bOffsH0,
+                                int bOffsW0, int bSzH, int bSzW, int bStrH, int bStrW, int numActive,
+                                const int16_t* activeBlockIndices, int transpose, void* stream)
+{
+    const int32_t bsize[2] = {bSzH, bSzW}, bstride[2] = {bStrH, bStrW}, boffset[2] = {bOffsH0, bOffsW0};
+    if (numActive < 0) return SBNET_EINVAL_ARG;
+    if (numActive > 0 && (!x || !y || !activeBlockIndices)) return SBNET_EINVAL_ARG;
+    if (!geom_ok(N, H, W, C, bsize, bstride)) return SBNET_EINVAL_ARG;
+    const sbnet::Geom g = make_geom(N, H, W, C, bsize, bstride, boffset);
+    SBNET_HIP(sbnet::launch_gather(x, y, activeBlockIndices, numActive, g, transpose != 0,
+                                   static_cast<hipStream_t>(stream)));
+    return SBNET_OK;
+}
+
+int sbnet_sparse_scatter(const float* x, int32_t num_active, const int16_t* active_block_indices,
+                         const float* ybase, const int64_t* ybase_dims, int ybase_rank,
+                         const int32_t* bsize, int bsize_len, const int32_t* bstride, int bstride_len,
+                         const int32_t* boffset, int boffset_len, int add, int atomic, int transpose,
+                         float* y, void* stream)
+{
+    // order of checks as in sparse_gather.cc:307-327
+    if (!pair_ok(bsize, bsize_len) || !pair_ok(bstride, bstride_len) || !pair_ok(boffset, boffset_len))
+        return SBNET_EINVAL_PARAM_SHAPE;
+    if (!atomic && add && !(bstride[0] >= bsize[0] && bstride[1] >= bsize[1])) return SBNET_EINVAL_OVERLAP;
+    if (ybase_rank != 4) return SBNET_EINVAL_RANK;
+    if (!ybase || !y || !ybase_dims || !dims_fit_int(ybase_dims)) return SBNET_EINVAL_ARG;
+    const size_t count = (size_t)ybase_dims[0] * ybase_dims[1] * ybase_dims[2] * ybase_dims[3];
+    {
+        const uintptr_t a = reinterpret_cast<uintptr_t>(ybase), b = reinterpret_cast<uintptr_t>(y);
+        const uintptr_t bytes = count * sizeof(float);
+        if (a < b + bytes && b < a + bytes) return SBNET_EINVAL_ARG;
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (!geom_ok((int)ybase_dims[0], (int)ybase_dims[1], (int)ybase_dims[2], (int)ybase_dims[3], bsize, bstride))
+        return SBNET_EINVAL_ARG;
+    SBNET_HIP(sbnet::launch_copy(y, ybase, count, s));  // sparse_gather.cc:338-346, no stream sync
+    return scatter_impl(x, num_active, active_block_indices, y, ybase_dims, bsize, bstride, boffset, add,
+                        atomic, transpose, s);
+}
+
+int sbnet_sparse_scatter_var(const float* x, int32_t num_active, const int16_t* active_block_indices,
+                             float* ybase, const int64_t* ybase_dims, int ybase_rank,
+                             const int32_t* bsize, int bsize_len, const int32_t* bstride,
+                             int bstride_len, const int32_t* boffset, int boffset_len, int add,
+                             int atomic, int transpose, void* stream)
+{
+    if (!pair_ok(bsize, bsize_len) || !pair_ok(bstride, bstride_len) || !pair_ok(boffset, boffset_len))
+        return SBNET_EINVAL_PARAM_SHAPE;
+    if (!atomic && add && !(bstride[0] >= bsize[0] && bstride[1] >= bsize[1])) return SBNET_EINVAL_OVERLAP;
+    if (ybase_rank != 4) return SBNET_EINVAL_RANK;
+    if (!ybase || !ybase_dims) return SBNET_EINVAL_ARG;
+    return scatter_impl(x, num_active, active_block_indices, ybase, ybase_dims, bsize, bstride, boffset,
+                        add, atomic, transpose, static_cast<hipStream_t>(stream));
+}
+
+int sbnet_sparse_scatter_functor(const float* x, int N, int H, int W, int C, float* y, int bOffsH0,
+                                 int bOffsW0, int bSzH, int bSzW, int bStrH, int bStrW, int numActive,
+                                 const int16_t* activeBlockIndices, int add, int transpose, int atomic,
+                                 void* stream)
+{
+    const int32_t bsize[2] = {bSzH, bSzW}, bstride[2] = {bStrH, bStrW}, boffset[2] = {bOffsH0, bOffsW0};
+    const int64_t dims[4] = {N, H, W, C};
+    return scatter_impl(x, numActive, activeBlockIndices, y, dims, bsize, bstride, boffset, add, atomic,
+                        transpose, static_cast<hipStream_t>(stream));
+}
+
+int sbnet_copy_tensor(float* dst, const float* src, size_t count, void* stream)
+{
+    if (count && (!dst || !src)) return SBNET_EINVAL_ARG;
+    SBNET_HIP(sbnet::launch_copy(dst, src, count, static_cast<hipStream_t>(stream)));
+    return SBNET_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,38 @@
+// Host-side launch interface between the C ABI (sbnet_capi.cpp) and the gfx950 kernels
+// (sbnet_kernels.hip).  Everything here takes already-validated arguments.
+#pragma once
+
+#include <hip/hip_runtime_api.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace sbnet {
+
+// Block geometry shared by the three ops.  Block (n, bh, bw) covers
+// x[n, oh + U*bh : oh + U*bh + R, ow + V*bw : ow + V*bw + S, :].
+struct Geom {
+    int N, H, W, C;
+    int R, S;    // block size  (bsize)
+    int U, V;    // block stride (bstride)
+    int oh, ow;  // block offset (boffset)
+};
+
+enum ScatterMode { SCATTER_ASSIGN = 0, SCATTER_ADD = 1, SCATTER_ATOMIC = 2 };
+
+// reduce_mask scratch layout: one flag byte per sparsity block, then one int32 count per
+// pooling workgroup, then one int32 for the total when the caller gives no device count.
+size_t reduce_mask_workspace_bytes(int64_t totalBlocks);
+
+hipError_t launch_reduce_mask(const float* mask, const Geom& g, int bCntH, int bCntW, float tol,
+                              bool avgPool, bool fixupZero, int16_t* activeBlockIndices,
+                              int32_t* binCountDevice, void* workspace, hipStream_t stream);
+
+hipError_t launch_gather(const float* x, float* y, const int16_t* idx, int numActive,
+                         const Geom& g, bool transpose, hipStream_t stream);
+
+hipError_t launch_scatter(const float* x, float* y, const int16_t* idx, int numActive,
+                          const Geom& g, bool transpose, ScatterMode mode, hipStream_t stream);
+
+hipError_t launch_copy(float* dst, const float* src, size_t count, hipStream_t stream);
+
+}  // namespace sbnet

@@ -1,0 +1,186 @@
+"""Host-side mirror of the reference's op interface over the C ABI of libsbnet_amd.so.
+
+The reference exposes its ops through `tf.load_op_library` as
+`sbnet_module.reduce_mask / sparse_gather / sparse_scatter / sparse_scatter_var`
+(sbnet_tensorflow/benchmark/sparse_conv_lib.py:74, 452-459, 547-554, 564-586; op signatures in
+sbnet_tensorflow/sbnet_ops/reduce_mask.cc:100-110 and sparse_gather.cc:48-57, 242-268).  The
+functions here keep those names, argument names and meanings.  PyTorch supplies device memory and
+the current stream only; all computation happens in the HIP kernels behind the C ABI, and there is
+no fallback if the library is missing.
+"""
+import collections
+import ctypes
+
+import numpy as np
+import torch
+
+from . import _lib
+
+ReduceMaskResult = collections.namedtuple("ReduceMask", ["active_block_indices", "bin_counts"])
+
+
+class InvalidArgument(ValueError):
+    """The reference ops fail with tensorflow's InvalidArgument status; same texts here."""
+
+
+class HipError(RuntimeError):
+    pass
+
+
+def _check(status):
+    if status == _lib.SBNET_OK:
+        return
+    lib = _lib.load()
+    text = lib.sbnet_status_string(status).decode()
+    if status == _lib.SBNET_EHIP:
+        raise HipError("%s: hipError_t %d" % (text, lib.sbnet_last_hip_error()))
+    raise InvalidArgument(text)
+
+
+def _pair(v):
+    """Host int32 parameter vector as (keepalive array, pointer, length); length is checked by the library."""
+    if isinstance(v, torch.Tensor):
+        v = v.detach().cpu().numpy()
+    a = np.ascontiguousarray(np.asarray(v, dtype=np.int32).reshape(-1))
+    return a, a.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)), int(a.shape[0])
+
+
+def _dims(t):
+    d = list(t.shape) + [1] * max(0, 4 - t.dim())
+    a = (ctypes.c_int64 * len(d))(*d)
+    return a, t.dim()
+
+
+def _dev_f32(t, name):
+    if not isinstance(t, torch.Tensor) or not t.is_cuda or t.dtype != torch.float32:
+        raise TypeError("%s must be a float32 tensor on the GPU" % name)
+    return t.contiguous()
+
+
+def _idx_i16(t):
+    if not isinstance(t, torch.Tensor) or not t.is_cuda or t.dtype != torch.int16:
+        raise TypeError("active_block_indices must be an int16 tensor on the GPU")
+    return t.contiguous()
+
+
+def _count(bin_counts):
+    """bin_counts lives in host memory in the reference (reduce_mask.cc:244, sparse_gather.cc:234)."""
+    if isinstance(bin_counts, torch.Tensor):
+        return int(bin_counts.reshape(-1)[0].item())
+    return int(np.asarray(bin_counts).reshape(-1)[0])
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+_workspaces = {}
+
+
+def _workspace(device, nbytes):
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1 << 16), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def reduce_mask(mask, dynamic_bcount, dynamic_bsize, dynamic_bstride, dynamic_boffset, tol, avgpool=False,
+                sync=True):
+    """ReduceMask (reduce_mask.cc:100-221).
+
+    mask: float32 GPU tensor [N,H,W,1] or [N,H,W].  Returns (active_block_indices, bin_counts):
+    int16 GPU tensor [N*bcount[0]*bcount[1], 3] whose first bin_counts[0] rows are the active blocks
+    in (n, bh, bw) lexicographic order, and an int32 tensor [1] in host memory.  With sync=False the
+    count is left on the device (bin_counts is then a GPU tensor) and the call does not wait.
+    """
+    lib = _lib.load()
+    mask = _dev_f32(mask, "mask")
+    if mask.dim() < 3:
+        raise InvalidArgument("mask must be [N,H,W,1]")
+    N, H, W = int(mask.shape[0]), int(mask.shape[1]), int(mask.shape[2])
+    bc, bcp, bcl = _pair(dynamic_bcount)
+    bs, bsp, bsl = _pair(dynamic_bsize)
+    bt, btp, btl = _pair(dynamic_bstride)
+    bo, bop, bol = _pair(dynamic_boffset)
+    max_idx = lib.sbnet_reduce_mask_max_indices(N, bcp, bcl) if bcl == 2 else 0
+    with torch.cuda.device(mask.device):
+        idx = torch.empty((max(int(max_idx), 1), 3), dtype=torch.int16, device=mask.device)
+        nws = lib.sbnet_reduce_mask_workspace_bytes(N, bcp, bcl) if bcl == 2 else 0
+        ws = _workspace(mask.device, nws)
+        dev_count = torch.empty(1, dtype=torch.int32, device=mask.device)
+        host_count = np.zeros(1, dtype=np.int32)
+        hp = host_count.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)) if sync else None
+        _check(lib.sbnet_reduce_mask(mask.data_ptr(), N, H, W, bcp, bcl, bsp, bsl, btp, btl, bop, bol,
+                                     ctypes.c_float(tol), int(bool(avgpool)), idx.data_ptr(), hp,
+                                     dev_count.data_ptr(), ws.data_ptr(), ws.numel(), _stream()))
+    if sync:
+        return ReduceMaskResult(idx, torch.from_numpy(host_count))
+    return ReduceMaskResult(idx, dev_count)
+
+
+def sparse_gather(x, bin_counts, active_block_indices, dynamic_bsize, dynamic_bstride, dynamic_boffset,
+                  transpose=False, out=None):
+    """SparseGather (sparse_gather.cc:48-57, 160-218): x [N,H,W,C] -> [M,bsize[0],bsize[1],C], or
+    [M,C,bsize[0],bsize[1]] with transpose=True, M = bin_counts[0]; out-of-image pixels read as 0."""
+    lib = _lib.load()
+    x = _dev_f32(x, "x")
+    idx = _idx_i16(active_block_indices)
+    M = _count(bin_counts)
+    bs, bsp, bsl = _pair(dynamic_bsize)
+    bt, btp, btl = _pair(dynamic_bstride)
+    bo, bop, bol = _pair(dynamic_boffset)
+    dims, rank = _dims(x)
+    y = out
+    with torch.cuda.device(x.device):
+        if y is None and rank == 4 and bsl == 2:
+            C, R, S = int(x.shape[3]), int(bs[0]), int(bs[1])
+            shape = (M, C, R, S) if transpose else (M, R, S, C)
+            y = torch.empty(shape, dtype=torch.float32, device=x.device)
+        _check(lib.sbnet_sparse_gather(x.data_ptr(), dims, rank, M, idx.data_ptr(), bsp, bsl, btp, btl, bop, bol,
+                                       int(bool(transpose)), y.data_ptr() if y is not None else None, _stream()))
+    return y
+
+
+def _scatter(x, bin_counts, active_block_indices, ybase, dynamic_bsize, dynamic_bstride, dynamic_boffset, add,
+             atomic, transpose, use_var):
+    lib = _lib.load()
+    x = _dev_f32(x, "x")
+    idx = _idx_i16(active_block_indices)
+    M = _count(bin_counts)
+    if not isinstance(ybase, torch.Tensor) or not ybase.is_cuda or ybase.dtype != torch.float32:
+        raise TypeError("ybase must be a float32 tensor on the GPU")
+    if use_var and not ybase.is_contiguous():
+        raise TypeError("sparse_scatter_var writes in place and needs a contiguous ybase")
+    ybase = ybase.contiguous()
+    bs, bsp, bsl = _pair(dynamic_bsize)
+    bt, btp, btl = _pair(dynamic_bstride)
+    bo, bop, bol = _pair(dynamic_boffset)
+    dims, rank = _dims(ybase)
+    with torch.cuda.device(ybase.device):
+        if use_var:
+            _check(lib.sbnet_sparse_scatter_var(x.data_ptr(), M, idx.data_ptr(), ybase.data_ptr(), dims, rank,
+                                                bsp, bsl, btp, btl, bop, bol, int(bool(add)), int(bool(atomic)),
+                                                int(bool(transpose)), _stream()))
+            return ybase
+        y = torch.empty_like(ybase)
+        _check(lib.sbnet_sparse_scatter(x.data_ptr(), M, idx.data_ptr(), ybase.data_ptr(), dims, rank, bsp, bsl,
+                                        btp, btl, bop, bol, int(bool(add)), int(bool(atomic)),
+                                        int(bool(transpose)), y.data_ptr(), _stream()))
+        return y
+
+
+def sparse_scatter(x, bin_counts, active_block_indices, ybase, dynamic_bsize, dynamic_bstride, dynamic_boffset,
+                   add, atomic=False, transpose=False):
+    """SparseScatter (sparse_gather.cc:256-268, 286-357): returns copy(ybase) with the blocks of x written
+    (add=False), added (add=True) or atomically added (add=True, atomic=True) on top."""
+    return _scatter(x, bin_counts, active_block_indices, ybase, dynamic_bsize, dynamic_bstride, dynamic_boffset,
+                    add, atomic, transpose, use_var=False)
+
+
+def sparse_scatter_var(x, bin_counts, active_block_indices, ybase, dynamic_bsize, dynamic_bstride,
+                       dynamic_boffset, add, atomic=False, transpose=False):
+    """SparseScatterVar (sparse_gather.cc:242-254, 335-337): the same, in place on ybase, which is returned."""
+    return _scatter(x, bin_counts, active_block_indices, ybase, dynamic_bsize, dynamic_bstride, dynamic_boffset,
+                    add, atomic, transpose, use_var=True)

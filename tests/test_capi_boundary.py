@@ -1,0 +1,131 @@
+"""The C-ABI boundary on a machine without a GPU: the library loads, exports every symbol that
+include/sbnet_amd.h declares, and returns the reference's InvalidArgument conditions before any
+device work (reduce_mask.cc:132-138; sparse_gather.cc:164-175, 307-327).  No kernel is launched here."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from sbnet_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+I32x2 = ctypes.c_int32 * 2
+I32x3 = ctypes.c_int32 * 3
+I64x4 = ctypes.c_int64 * 4
+FAKE = ctypes.c_void_p(0x1000)  # never dereferenced: every call below fails validation first
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "sbnet_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sbnet_[a-z_]+)\s*\(", text)))
+
+
+def test_header_declares_what_the_loader_binds():
+    assert declared_symbols() == sorted(_lib.SIGNATURES)
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared_symbols():
+        assert hasattr(lib, name), name
+
+
+def test_version_and_status_strings():
+    lib = _lib.load()
+    assert b"gfx950" in lib.sbnet_version()
+    assert b"one-dimensional with shape[0] == 2" in lib.sbnet_status_string(_lib.SBNET_EINVAL_PARAM_SHAPE)
+    assert b"Only non-overlapping blocks are supported with add=True, atomic=False" in \
+        lib.sbnet_status_string(_lib.SBNET_EINVAL_OVERLAP)
+    assert b"rank 4" in lib.sbnet_status_string(_lib.SBNET_EINVAL_RANK)
+    assert lib.sbnet_status_string(_lib.SBNET_OK) == b"OK"
+
+
+def test_size_queries():
+    lib = _lib.load()
+    assert lib.sbnet_reduce_mask_max_indices(4, I32x2(16, 16), 2) == 1024  # reduce_mask.cc:161
+    assert lib.sbnet_reduce_mask_max_indices(4, I32x3(16, 16, 1), 3) == -1
+    assert lib.sbnet_reduce_mask_workspace_bytes(4, I32x2(16, 16), 2) >= 1024
+    assert lib.sbnet_reduce_mask_workspace_bytes(4, I32x3(1, 1, 1), 3) == 0
+
+
+def test_reduce_mask_param_shape_errors():
+    lib = _lib.load()
+    ok = I32x2(2, 2)
+    bad = I32x3(2, 2, 2)
+    for pos in range(4):
+        ptrs = [ok, ok, ok, ok]
+        lens = [2, 2, 2, 2]
+        ptrs[pos], lens[pos] = bad, 3
+        rc = lib.sbnet_reduce_mask(FAKE, 1, 4, 4, ptrs[0], lens[0], ptrs[1], lens[1], ptrs[2], lens[2], ptrs[3],
+                                   lens[3], 0.5, 0, FAKE, None, FAKE, None, 0, None)
+        assert rc == _lib.SBNET_EINVAL_PARAM_SHAPE
+    # arguments the reference never checks but that would fault a kernel
+    rc = lib.sbnet_reduce_mask(None, 1, 4, 4, ok, 2, ok, 2, ok, 2, ok, 2, 0.5, 0, FAKE, None, FAKE, None, 0, None)
+    assert rc == _lib.SBNET_EINVAL_ARG
+    rc = lib.sbnet_reduce_mask(FAKE, 1, 4, 4, ok, 2, ok, 2, ok, 2, ok, 2, 0.5, 0, FAKE, None, None, None, 0, None)
+    assert rc == _lib.SBNET_EINVAL_ARG  # no count destination at all
+    rc = lib.sbnet_reduce_mask(FAKE, 1, 4, 4, I32x2(40000, 2), 2, ok, 2, ok, 2, ok, 2, 0.5, 0, FAKE, None, FAKE,
+                               None, 0, None)
+    assert rc == _lib.SBNET_EINVAL_ARG  # bh would not fit the int16 index triple
+    rc = lib.sbnet_reduce_mask(FAKE, 1, 4, 4, ok, 2, ok, 2, ok, 2, ok, 2, 0.5, 0, FAKE, None, FAKE, FAKE, 8, None)
+    assert rc == _lib.SBNET_EINVAL_ARG  # workspace too small
+    rc = lib.sbnet_reduce_mask_functor(FAKE, 1, 4, 4, 0.5, 0, 0, 2, 2, 2, 2, 2, 2, 2, 2, FAKE, FAKE, 0, None, 0,
+                                       None)
+    assert rc == _lib.SBNET_EINVAL_ARG  # numBins must be 1 (reduce_mask.cc:69)
+
+
+def test_gather_errors():
+    lib = _lib.load()
+    ok = I32x2(2, 2)
+    dims = I64x4(1, 4, 4, 1)
+    assert lib.sbnet_sparse_gather(FAKE, dims, 3, 1, FAKE, ok, 2, ok, 2, ok, 2, 0, FAKE, None) == \
+        _lib.SBNET_EINVAL_RANK
+    assert lib.sbnet_sparse_gather(FAKE, dims, 4, 1, FAKE, ok, 2, I32x3(1, 1, 1), 3, ok, 2, 0, FAKE, None) == \
+        _lib.SBNET_EINVAL_PARAM_SHAPE
+    # rank is checked before the parameter vectors (sparse_gather.cc:164 then :169-175)
+    assert lib.sbnet_sparse_gather(FAKE, dims, 5, 1, FAKE, ok, 1, ok, 2, ok, 2, 0, FAKE, None) == \
+        _lib.SBNET_EINVAL_RANK
+    assert lib.sbnet_sparse_gather(FAKE, dims, 4, -1, FAKE, ok, 2, ok, 2, ok, 2, 0, FAKE, None) == \
+        _lib.SBNET_EINVAL_ARG
+    assert lib.sbnet_sparse_gather(FAKE, dims, 4, 1, None, ok, 2, ok, 2, ok, 2, 0, FAKE, None) == \
+        _lib.SBNET_EINVAL_ARG
+    # zero active blocks is a no-op, not an error
+    assert lib.sbnet_sparse_gather(FAKE, dims, 4, 0, None, ok, 2, ok, 2, ok, 2, 0, None, None) == _lib.SBNET_OK
+
+
+@pytest.mark.parametrize("var", [False, True])
+def test_scatter_errors(var):
+    lib = _lib.load()
+    dims = I64x4(1, 4, 4, 1)
+    size, overlap, ok = I32x2(2, 2), I32x2(1, 2), I32x2(2, 2)
+
+    def call(rank, bstride, blen, add, atomic):
+        if var:
+            return lib.sbnet_sparse_scatter_var(FAKE, 1, FAKE, FAKE, dims, rank, size, 2, bstride, blen, ok, 2, add,
+                                                atomic, 0, None)
+        return lib.sbnet_sparse_scatter(FAKE, 1, FAKE, FAKE, dims, rank, size, 2, bstride, blen, ok, 2, add, atomic,
+                                        0, ctypes.c_void_p(0x100000), None)
+
+    assert call(4, overlap, 2, 1, 0) == _lib.SBNET_EINVAL_OVERLAP      # sparse_gather.cc:322-326
+    assert call(3, overlap, 2, 1, 0) == _lib.SBNET_EINVAL_OVERLAP      # tested before the rank
+    assert call(3, overlap, 2, 1, 1) == _lib.SBNET_EINVAL_RANK         # sparse_gather.cc:327
+    assert call(3, overlap, 2, 0, 0) == _lib.SBNET_EINVAL_RANK
+    assert call(4, I32x3(2, 2, 2), 3, 0, 0) == _lib.SBNET_EINVAL_PARAM_SHAPE  # sparse_gather.cc:307-313
+
+
+def test_scatter_rejects_aliasing_output():
+    lib = _lib.load()
+    dims = I64x4(1, 4, 4, 1)
+    ok = I32x2(2, 2)
+    rc = lib.sbnet_sparse_scatter(FAKE, 1, FAKE, FAKE, dims, 4, ok, 2, ok, 2, ok, 2, 0, 0, 0,
+                                  ctypes.c_void_p(0x1000 + 16), None)
+    assert rc == _lib.SBNET_EINVAL_ARG
+
+
+def test_python_mirror_fails_loudly_without_library(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libsbnet_amd.so")
+    with pytest.raises(RuntimeError, match="no CPU or PyTorch fallback"):
+        _lib.load()

@@ -1,0 +1,482 @@
+"""Parity of the HIP kernels (through the C ABI, via sbnet_amd.ops) with the CPU oracle.
+
+Bars: active-block lists and bin_counts bit-exact *including order* (the kernels write the CPU
+functor's lexicographic order); gather and non-atomic scatter bit-exact in fp32; atomic
+scatter-add on overlapping blocks within 1e-6 relative (tolerance defined in `assert_atomic_close`).
+
+The case menu is the reference's own (sbnet_ops/tests/test_sparse_blocks.py:345-449) plus the five
+benchmark configurations at full size and the hand-written vectors of tests/golden.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import sbnet_amd
+from sbnet_amd import workloads
+from closed_forms import box_sum_valid
+from oracle import sbnet_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+with open(os.path.join(HERE, "golden", "known_answers.json")) as f:
+    GOLD = json.load(f)
+
+DEV = "cuda:0"
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def host(t):
+    return t.detach().cpu().numpy()
+
+
+def bcount_covering(H, W, bstride, boffset):
+    return [1 + (H - boffset[0] - 1) // bstride[0], 1 + (W - boffset[1] - 1) // bstride[1]]
+
+
+def assert_atomic_close(got, exp):
+    """|got - exp| <= 1e-6 * max(|exp|, 1e-6 * max|exp|), the "1e-6 relative" bar for atomic adds;
+    a few addends per pixel can only differ from the sequential sum by fp32 reassociation."""
+    scale = np.maximum(np.abs(exp), 1e-6 * float(np.abs(exp).max() if exp.size else 0.0))
+    bad = np.abs(got - exp) > 1e-6 * scale
+    assert not bad.any(), "max rel err %g" % float((np.abs(got - exp) / np.maximum(scale, 1e-30)).max())
+
+
+def check_reduce(mask, bc, bs, bst, bo, tol, avgpool):
+    """Runs reduce_mask on both sides, asserts equality and returns (host idx, host count, device idx)."""
+    idx_o, cnt_o = orc.reduce_mask(mask, bc, bs, bst, bo, tol, avgpool)
+    r = sbnet_amd.reduce_mask(dev(mask), bc, bs, bst, bo, tol=tol, avgpool=avgpool)
+    assert r.bin_counts.dtype == torch.int32 and not r.bin_counts.is_cuda
+    M = int(cnt_o[0])
+    assert int(r.bin_counts[0]) == M
+    assert r.active_block_indices.shape == (mask.shape[0] * bc[0] * bc[1], 3)
+    np.testing.assert_array_equal(host(r.active_block_indices)[:M], idx_o[:M])
+    return idx_o, cnt_o, r
+
+
+def run_case(shape, RS, UV, BOFFS=(-1, -2), sparsity=70, do_add=False, N=1, test_var=False, avgpool=False,
+             use_atomics=False, seed=0):
+    """One runTestForOneSize of the reference's integration test, both transposes."""
+    H, W, C = shape
+    rng = np.random.default_rng(seed)
+    bc = bcount_covering(H, W, UV, BOFFS)
+    mask = rng.standard_normal((N, H, W, 1)).astype(np.float32)
+    x = rng.standard_normal((N, H, W, C)).astype(np.float32)
+    tol = float(np.percentile(x, sparsity)) if sparsity != 100 else 1e32
+    idx_o, cnt_o, r = check_reduce(mask, bc, RS, UV, BOFFS, tol, avgpool)
+    if sparsity == 100:
+        assert int(cnt_o[0]) == 1 and idx_o[0].tolist() == [0, 0, 0]
+    xd = dev(x)
+    base = (x * 0.0 + 10.0).astype(np.float32)
+    overlap = UV[0] < RS[0] or UV[1] < RS[1]
+    g_ut = None
+    for transpose in (False, True):
+        g_o = orc.sparse_gather(x, cnt_o, idx_o, RS, UV, BOFFS, transpose=transpose)
+        g = sbnet_amd.sparse_gather(xd, r.bin_counts, r.active_block_indices, RS, UV, BOFFS, transpose=transpose)
+        assert tuple(g.shape) == g_o.shape
+        np.testing.assert_array_equal(host(g), g_o)
+        if not transpose:
+            g_ut = g_o
+        else:
+            np.testing.assert_array_equal(host(g), g_ut.transpose(0, 3, 1, 2))
+        if do_add and overlap and not use_atomics:
+            continue
+        y_o = orc.sparse_scatter(g_o, cnt_o, idx_o, base, RS, UV, BOFFS, add=do_add, atomic=use_atomics,
+                                 transpose=transpose)
+        bd = dev(base)
+        fn = sbnet_amd.sparse_scatter_var if test_var else sbnet_amd.sparse_scatter
+        y = fn(g, r.bin_counts, r.active_block_indices, bd, RS, UV, BOFFS, add=do_add, atomic=use_atomics,
+               transpose=transpose)
+        if test_var:
+            assert y.data_ptr() == bd.data_ptr()
+        else:
+            np.testing.assert_array_equal(host(bd), base)  # the copying op leaves ybase alone
+        if do_add and use_atomics and overlap:
+            assert_atomic_close(host(y), y_o)
+        else:
+            # add=False on overlaps writes equal values from every covering block, so order cannot matter
+            np.testing.assert_array_equal(host(y), y_o)
+
+
+# ---------------------------------------------------------------------------------------------
+# golden vectors
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("case", GOLD["reduce_mask"], ids=lambda c: c["name"])
+def test_reduce_mask_golden(case):
+    mask = np.asarray(case["mask"], np.float32)[None, :, :, None]
+    r = sbnet_amd.reduce_mask(dev(mask), case["bcount"], case["bsize"], case["bstride"], case["boffset"],
+                              tol=case["tol"], avgpool=case["avgpool"])
+    M = int(r.bin_counts[0])
+    assert host(r.active_block_indices)[:M].tolist() == case["expected_indices"]
+
+
+@pytest.mark.parametrize("case", GOLD["gather_arange"], ids=lambda c: c["name"])
+def test_gather_arange_golden(case):
+    H, W = case["shape"]
+    x = np.arange(H * W, dtype=np.float32).reshape(1, H, W, 1)
+    idx = np.asarray(case["indices"], np.int16)
+    y = sbnet_amd.sparse_gather(dev(x), [len(idx)], dev(idx), case["bsize"], case["bstride"], case["boffset"])
+    assert host(y).reshape(len(idx), -1).tolist() == case["expected_blocks"]
+
+
+@pytest.mark.parametrize("use_var", [False, True])
+@pytest.mark.parametrize("transpose", [False, True])
+@pytest.mark.parametrize("case", GOLD["pipeline"], ids=lambda c: c["name"])
+def test_pipeline_known_answers(case, transpose, use_var):
+    mask = np.asarray(case["mask"], np.float32)[None, :, :, None]
+    x = np.ones_like(mask)
+    r = sbnet_amd.reduce_mask(dev(mask), case["bcount"], case["bsize"], case["bstride"], case["boffset"], tol=0.0)
+    p = sbnet_amd.sparse_gather(dev(x), r.bin_counts, r.active_block_indices, case["bsize"], case["bstride"],
+                                case["boffset"], transpose=transpose)
+    p = host(p)
+    q = box_sum_valid(p.transpose(0, 2, 3, 1) if transpose else p, case["ksize"][0], case["ksize"][1])
+    if transpose:
+        q = np.ascontiguousarray(q.transpose(0, 3, 1, 2))
+    y_exp = np.asarray(case["y_exp"], np.float32)[None, :, :, None]
+    fn = sbnet_amd.sparse_scatter_var if use_var else sbnet_amd.sparse_scatter
+    y = fn(dev(q), r.bin_counts, r.active_block_indices, dev(np.zeros_like(y_exp)), case["bsize_out"],
+           case["bstride"], [0, 0], add=False, transpose=transpose)
+    np.testing.assert_array_equal(host(y), y_exp)
+
+
+# ---------------------------------------------------------------------------------------------
+# the reference integration test's case list
+# ---------------------------------------------------------------------------------------------
+
+def test_simple():
+    run_case((2, 3, 2), RS=(2, 3), UV=(3, 4))
+    run_case((5, 5, 1), RS=(3, 3), UV=(1, 1))
+
+
+def test_zero_block_count():
+    run_case((2, 2, 1), RS=(1, 1), UV=(1, 1), BOFFS=(0, 0), sparsity=100)
+    run_case((40, 40, 8), RS=(5, 5), UV=(5, 5), BOFFS=(0, 0), sparsity=100, avgpool=True, N=3)
+
+
+def test_basic_and_overlapping():
+    run_case((2, 2, 1), RS=(1, 1), UV=(1, 1), BOFFS=(0, 0), sparsity=0)
+    run_case((2, 2, 1), RS=(1, 1), UV=(1, 1), BOFFS=(0, 0), sparsity=0, N=3)
+    run_case((6, 6, 1), RS=(1, 1), UV=(1, 1))
+    run_case((3, 3, 1), RS=(2, 2), UV=(1, 1), BOFFS=(0, 0), sparsity=0)
+    run_case((13, 12, 1), RS=(2, 3), UV=(1, 2), BOFFS=(0, 0), sparsity=0.1)
+
+
+@pytest.mark.parametrize("sparsity", [10, 20, 30, 40, 50, 70, 90, 99])
+def test_sparsities(sparsity):
+    # avg pooling over a Gaussian (non-binary) mask: decisions must follow the CPU summation order
+    run_case((200, 300, 32), RS=(3, 4), UV=(2, 3), sparsity=sparsity, avgpool=True, use_atomics=True)
+
+
+def test_avg_pooling_with_holes():
+    run_case((2, 3, 2), RS=(2, 3), UV=(3, 4), avgpool=True)
+    run_case((2, 3, 2), RS=(2, 3), UV=(3, 4), avgpool=False)
+
+
+@pytest.mark.parametrize("cc", [15, 16, 24, 32, 48, 64])
+def test_channel_sweep(cc):
+    run_case((380, 480, cc), RS=(18, 18), UV=(18, 18))
+
+
+def test_channel_sweep_16():
+    run_case((200, 300, 32), RS=(16, 16), UV=(16, 16))
+
+
+@pytest.mark.parametrize("avgpool", [True, False])
+@pytest.mark.parametrize("tv", [True, False])
+@pytest.mark.parametrize("nn", [1, 7])
+def test_simple_permutations(nn, tv, avgpool):
+    for sp in [0, 10, 50, 99]:
+        args = dict(RS=(1, 1), UV=(1, 1), BOFFS=[0, 0], sparsity=sp, N=nn, test_var=tv, avgpool=avgpool)
+        for shape in [(1, 1, 1), (1, 1, 2), (1, 2, 3), (2, 1, 3), (3, 2, 1), (1, 2, 1), (3, 2, 7)]:
+            run_case(shape, **args)
+    run_case((1, 1, 1024 * 49), RS=(1, 1), UV=(1, 1), BOFFS=[0, 0], sparsity=50, N=nn, test_var=tv,
+             avgpool=avgpool)
+
+
+def test_uneven_gaps_offsets():
+    run_case((8, 10, 7), RS=(3, 4), UV=(3, 4))
+    run_case((8, 10, 1), RS=(3, 4), UV=(4, 5))
+    run_case((8, 10, 7), RS=(3, 4), UV=(4, 5))
+    run_case((5, 5, 1), RS=(3, 2), UV=(3, 2), BOFFS=[-1, -2])
+    run_case((5, 3, 1), RS=(2, 3), UV=(2, 3), BOFFS=[0, 0])
+    run_case((5, 3, 1), RS=(2, 3), UV=(2, 3), BOFFS=[-1, -2])
+    run_case((3, 3, 1), RS=(2, 2), UV=(1, 1), BOFFS=[0, 0])
+    run_case((3, 3, 1), RS=(1, 1), UV=(2, 2))
+
+
+def test_large_block_sizes():
+    run_case((2048, 2048, 1), RS=(1500, 490), UV=(300, 390), use_atomics=True)
+
+
+@pytest.mark.parametrize("C", [1, 2, 3, 6, 7, 12, 20, 128, 130])
+@pytest.mark.parametrize("do_add", [False, True])
+def test_odd_channels_and_adds(C, do_add):
+    run_case((33, 47, C), RS=(5, 7), UV=(5, 7), BOFFS=(-2, -3), sparsity=40, do_add=do_add, N=2, seed=C)
+    run_case((33, 47, C), RS=(5, 7), UV=(3, 4), BOFFS=(-2, -3), sparsity=40, do_add=do_add, N=2,
+             use_atomics=True, seed=C + 100)
+
+
+def test_misaligned_base_pointers():
+    """Tensors whose storage starts 4 or 8 bytes past a 16-byte boundary take the narrower vector paths."""
+    rng = np.random.default_rng(21)
+    N, H, W, C = 2, 20, 24, 8
+    bs, bst, bo = (5, 6), (5, 6), (-1, -1)
+    bc = bcount_covering(H, W, bst, bo)
+    x = rng.standard_normal((N, H, W, C)).astype(np.float32)
+    mask = rng.standard_normal((N, H, W, 1)).astype(np.float32)
+    idx_o, cnt_o, r = check_reduce(mask, bc, bs, bst, bo, 0.2, False)
+    for off in (1, 2, 3):
+        buf = torch.zeros(x.size + 8, dtype=torch.float32, device=DEV)
+        xd = buf[off:off + x.size].view(N, H, W, C)
+        xd.copy_(torch.from_numpy(x))
+        assert xd.data_ptr() % 16 == 4 * off
+        for transpose in (False, True):
+            g_o = orc.sparse_gather(x, cnt_o, idx_o, bs, bst, bo, transpose=transpose)
+            gbuf = torch.zeros(g_o.size + 8, dtype=torch.float32, device=DEV)
+            gout = gbuf[off:off + g_o.size].view(*g_o.shape)
+            sbnet_amd.sparse_gather(xd, r.bin_counts, r.active_block_indices, bs, bst, bo, transpose=transpose,
+                                    out=gout)
+            np.testing.assert_array_equal(host(gout), g_o)
+            ybuf = torch.full((x.size + 8,), 10.0, dtype=torch.float32, device=DEV)
+            yd = ybuf[off:off + x.size].view(N, H, W, C)
+            sbnet_amd.sparse_scatter_var(gout, r.bin_counts, r.active_block_indices, yd, bs, bst, bo, add=True,
+                                         transpose=transpose)
+            y_o = orc.sparse_scatter(g_o, cnt_o, idx_o, np.full_like(x, 10.0), bs, bst, bo, add=True,
+                                     transpose=transpose)
+            np.testing.assert_array_equal(host(yd), y_o)
+            assert float(ybuf[:off].min()) == 10.0 and float(ybuf[off + x.size:].max()) == 10.0
+
+
+# ---------------------------------------------------------------------------------------------
+# reduce_mask: summation order, thresholds, sizes
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("bs,bst", [((6, 6), (4, 4)), ((18, 18), (16, 16)), ((27, 27), (25, 25)), ((3, 50), (3, 45)),
+                                    ((64, 2), (60, 2)), ((40, 40), (10, 10))])
+def test_reduce_mask_avg_order_sensitive(bs, bst):
+    """Masks built so that fp32 summation order changes block sums, with thresholds sitting on the
+    sequential sums themselves: any deviation from the row-major order flips decisions."""
+    rng = np.random.default_rng(bs[0] * 100 + bs[1])
+    N, H, W = 3, 160, 190
+    bo = (-1, -1)
+    bc = bcount_covering(H, W, bst, bo)
+    mask = (rng.standard_normal((N, H, W, 1)) * rng.choice([1e-3, 1.0, 1e4], size=(N, H, W, 1))).astype(np.float32)
+    # thresholds: the exact sequential average of a few blocks (ties) and values one ulp either side
+    sums = []
+    for n, bh, bw in [(0, 1, 1), (1, 2, 3), (2, 0, 0), (1, bc[0] - 1, bc[1] - 1)]:
+        h0, w0 = bo[0] + bh * bst[0], bo[1] + bw * bst[1]
+        s = np.float32(0)
+        for hh in range(max(h0, 0), min(h0 + bs[0], H)):
+            for ww in range(max(w0, 0), min(w0 + bs[1], W)):
+                s = np.float32(s + mask[n, hh, ww, 0])
+        sums.append(np.float32(s / np.float32(bs[0] * bs[1])))
+    for t in sums:
+        for tol in (t, np.nextafter(t, np.float32(-np.inf)), np.nextafter(t, np.float32(np.inf))):
+            check_reduce(mask, bc, bs, bst, bo, float(tol), True)
+    check_reduce(mask, bc, bs, bst, bo, 0.0, True)
+
+
+def test_reduce_mask_special_values():
+    rng = np.random.default_rng(5)
+    N, H, W = 2, 64, 64
+    bs, bst, bo = (9, 9), (8, 8), (-1, -1)
+    bc = [8, 8]
+    mask = rng.standard_normal((N, H, W, 1)).astype(np.float32)
+    mask[0, 3, 3, 0] = np.inf
+    mask[0, 20, 20, 0] = -np.inf
+    mask[0, 40, 40, 0] = np.nan
+    mask[1, 10, 10, 0] = np.inf
+    mask[1, 11, 11, 0] = -np.inf
+    mask[1, 50, 50, 0] = 3e38
+    mask[1, 51, 51, 0] = 3e38
+    for avg in (False, True):
+        for tol in (-1.0, 0.0, 0.05, 1e30):
+            check_reduce(mask, bc, bs, bst, bo, tol, avg)
+
+
+def test_reduce_mask_many_blocks_and_async_count():
+    rng = np.random.default_rng(8)
+    N, H, W = 5, 300, 300
+    mask = (rng.random((N, H, W, 1)) < 0.3).astype(np.float32)
+    bc = bcount_covering(H, W, (2, 2), (0, 0))
+    idx_o, cnt_o, r = check_reduce(mask, bc, (2, 2), (2, 2), (0, 0), 0.4, True)
+    r2 = sbnet_amd.reduce_mask(dev(mask), bc, (2, 2), (2, 2), (0, 0), tol=0.4, avgpool=True, sync=False)
+    assert r2.bin_counts.is_cuda
+    torch.cuda.synchronize()
+    assert int(r2.bin_counts[0]) == int(cnt_o[0])
+    np.testing.assert_array_equal(host(r2.active_block_indices)[:int(cnt_o[0])], idx_o[:int(cnt_o[0])])
+
+
+def test_reduce_mask_rows_past_count_untouched():
+    mask = np.zeros((1, 8, 8, 1), np.float32)
+    mask[0, 0, 0, 0] = 1.0
+    lib_idx = torch.full((16, 3), 77, dtype=torch.int16, device=DEV)
+    # call through the raw ABI with a caller-owned index buffer
+    import ctypes
+    from sbnet_amd import _lib
+    L = _lib.load()
+    I2 = ctypes.c_int32 * 2
+    nws = L.sbnet_reduce_mask_workspace_bytes(1, I2(4, 4), 2)
+    ws = torch.empty(nws, dtype=torch.uint8, device=DEV)
+    cnt = np.zeros(1, np.int32)
+    rc = L.sbnet_reduce_mask(dev(mask).data_ptr(), 1, 8, 8, I2(4, 4), 2, I2(2, 2), 2, I2(2, 2), 2, I2(0, 0), 2, 0.5,
+                             0, lib_idx.data_ptr(), cnt.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)), None,
+                             ws.data_ptr(), nws, None)
+    assert rc == 0 and cnt[0] == 1
+    out = host(lib_idx)
+    assert out[0].tolist() == [0, 0, 0] and (out[1:] == 77).all()
+    # without a workspace the library allocates its own
+    rc = L.sbnet_reduce_mask(dev(mask).data_ptr(), 1, 8, 8, I2(4, 4), 2, I2(2, 2), 2, I2(2, 2), 2, I2(0, 0), 2, 0.5,
+                             0, lib_idx.data_ptr(), cnt.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)), None,
+                             None, 0, None)
+    assert rc == 0 and cnt[0] == 1
+    # functor level: raw count, zero stays zero and nothing is written
+    lib_idx.fill_(55)
+    dcnt = torch.full((1,), -1, dtype=torch.int32, device=DEV)
+    rc = L.sbnet_reduce_mask_functor(dev(mask * 0).data_ptr(), 1, 8, 8, 0.5, 0, 0, 2, 2, 2, 2, 4, 4, 1, 16,
+                                     lib_idx.data_ptr(), dcnt.data_ptr(), 0, ws.data_ptr(), nws, None)
+    torch.cuda.synchronize()
+    assert rc == 0 and int(dcnt[0]) == 0 and (host(lib_idx) == 55).all()
+
+
+# ---------------------------------------------------------------------------------------------
+# functor-level entry points and the copy
+# ---------------------------------------------------------------------------------------------
+
+def test_functor_level_entry_points():
+    import ctypes
+    from sbnet_amd import _lib
+    L = _lib.load()
+    rng = np.random.default_rng(31)
+    N, H, W, C = 2, 30, 40, 12
+    R, S, U, V, oh, ow = 7, 5, 6, 5, -2, -1
+    bc = bcount_covering(H, W, (U, V), (oh, ow))
+    x = rng.standard_normal((N, H, W, C)).astype(np.float32)
+    mask = rng.standard_normal((N, H, W, 1)).astype(np.float32)
+    idx_o, cnt_o = orc.reduce_mask(mask, bc, (R, S), (U, V), (oh, ow), 0.5, False)
+    M = int(cnt_o[0])
+    idx_d = dev(idx_o)
+    xd = dev(x)
+    for transpose in (0, 1):
+        g_o = orc.sparse_gather(x, cnt_o, idx_o, (R, S), (U, V), (oh, ow), transpose=bool(transpose))
+        g = torch.empty(g_o.shape, dtype=torch.float32, device=DEV)
+        assert L.sbnet_sparse_gather_functor(xd.data_ptr(), N, H, W, C, g.data_ptr(), oh, ow, R, S, U, V, M,
+                                             idx_d.data_ptr(), transpose, None) == 0
+        np.testing.assert_array_equal(host(g), g_o)
+        base = rng.standard_normal((N, H, W, C)).astype(np.float32)
+        yd = dev(base)
+        assert L.sbnet_sparse_scatter_functor(g.data_ptr(), N, H, W, C, yd.data_ptr(), oh, ow, R, S, U, V, M,
+                                              idx_d.data_ptr(), 1, transpose, 1, None) == 0
+        y_o = orc.sparse_scatter(g_o, cnt_o, idx_o, base, (R, S), (U, V), (oh, ow), add=True, atomic=True,
+                                 transpose=bool(transpose))
+        assert_atomic_close(host(yd), y_o)
+    for count in (0, 1, 3, 4, 1023, 4096 + 5):
+        src = torch.arange(count + 3, dtype=torch.float32, device=DEV)
+        dst = torch.full((count + 3,), -1.0, device=DEV)
+        for off in (0, 1):
+            dst.fill_(-1.0)
+            assert L.sbnet_copy_tensor(dst.data_ptr() + 4 * off, src.data_ptr() + 4 * off, count, None) == 0
+            torch.cuda.synchronize()
+            assert torch.equal(dst[off:off + count], src[off:off + count])
+            assert float(dst[off + count:].max()) == -1.0
+
+
+# ---------------------------------------------------------------------------------------------
+# the five benchmark configurations at full size
+# ---------------------------------------------------------------------------------------------
+
+def run_workload(wl):
+    """reduce_mask -> gather -> (centre crop) -> scatter on a Workload, compared op by op."""
+    idx_o, cnt_o, r = check_reduce(wl.mask, wl.bcount, wl.bsize, wl.bstride, wl.boffset, wl.tol, wl.avgpool)
+    M = int(cnt_o[0])
+    xd = dev(wl.x)
+    g = sbnet_amd.sparse_gather(xd, r.bin_counts, r.active_block_indices, wl.bsize, wl.bstride, wl.boffset,
+                                transpose=wl.transpose)
+    g_o = orc.sparse_gather(wl.x, cnt_o, idx_o, wl.bsize, wl.bstride, wl.boffset, transpose=wl.transpose, omp=True)
+    np.testing.assert_array_equal(host(g), g_o)
+    q = workloads.centre_crop(g, wl.bsize, wl.s_bsize, wl.transpose).contiguous()
+    q_o = np.ascontiguousarray(workloads.centre_crop(g_o, wl.bsize, wl.s_bsize, wl.transpose))
+    base = np.zeros(wl.shape, np.float32) if wl.name == "C1" else wl.x
+    fn = sbnet_amd.sparse_scatter_var if wl.s_var else sbnet_amd.sparse_scatter
+    bd = dev(base)
+    y = fn(q, r.bin_counts, r.active_block_indices, bd, wl.s_bsize, wl.s_bstride, wl.s_boffset, add=wl.s_add,
+           atomic=wl.s_atomic, transpose=wl.transpose)
+    y_o = orc.sparse_scatter(q_o, cnt_o, idx_o, base, wl.s_bsize, wl.s_bstride, wl.s_boffset, add=wl.s_add,
+                             atomic=wl.s_atomic, transpose=wl.transpose)
+    np.testing.assert_array_equal(host(y), y_o)
+    return M
+
+
+def test_config1_plumbing():
+    c = GOLD["config1"]
+    wl = workloads.config1(c["seed"])
+    assert run_workload(wl) == len(c["expected_indices"])
+
+
+def test_config2_ellipses_avgpool():
+    assert run_workload(workloads.config2()) > 10
+
+
+@pytest.mark.parametrize("density", [0.05, 0.15, 0.30])
+def test_config3_bev(density):
+    wl = workloads.config3(density)
+    M = run_workload(wl)
+    assert abs(M / 1024.0 - density) < 0.03
+
+
+def test_config3_roundtrip_is_identity():
+    """scatter_var(gather(x)) with the gather geometry rewrites x with its own values: x is unchanged,
+    and scattering into zeros reproduces x exactly on the covered pixels (size-independent property)."""
+    wl = workloads.config3(0.30)
+    xd = dev(wl.x)
+    r = sbnet_amd.reduce_mask(dev(wl.mask), wl.bcount, wl.bsize, wl.bstride, wl.boffset, tol=wl.tol)
+    g = sbnet_amd.sparse_gather(xd, r.bin_counts, r.active_block_indices, wl.bsize, wl.bstride, wl.boffset,
+                                transpose=True)
+    keep = xd.clone()
+    sbnet_amd.sparse_scatter_var(g, r.bin_counts, r.active_block_indices, xd, wl.bsize, wl.bstride, wl.boffset,
+                                 add=False, transpose=True)
+    assert torch.equal(xd, keep)
+    z = torch.zeros_like(xd)
+    sbnet_amd.sparse_scatter_var(g, r.bin_counts, r.active_block_indices, z, wl.bsize, wl.bstride, wl.boffset,
+                                 add=False, transpose=True)
+    covered = z != 0
+    assert torch.equal(z[covered], xd[covered]) and 0.2 < float(covered.float().mean()) < 0.45
+
+
+def test_config4_overlapping_atomic_add():
+    wl = workloads.config4()
+    N, H, W, C = wl.shape
+    M = len(wl.indices)
+    gen = torch.Generator(device=DEV).manual_seed(1004)
+    stack = torch.rand((M, 16, 16, C), generator=gen, device=DEV) * 2.0 - 1.0
+    base = torch.zeros((N, H, W, C), device=DEV)
+    idx_d = dev(wl.indices)
+    out = sbnet_amd.sparse_scatter_var(stack, [M], idx_d, base, wl.s_bsize, wl.s_bstride, wl.s_boffset, add=True,
+                                       atomic=True)
+    assert out.data_ptr() == base.data_ptr()
+    y_o = np.zeros((N, H, W, C), np.float32)
+    orc.sparse_scatter_raw(host(stack), M, wl.indices, y_o, wl.s_bsize, wl.s_bstride, wl.s_boffset, add=True,
+                           transpose=False)
+    assert_atomic_close(host(base), y_o)
+    # linearity (size-independent): scattering the stack twice doubles the result exactly
+    sbnet_amd.sparse_scatter_var(stack, [M], idx_d, base, wl.s_bsize, wl.s_bstride, wl.s_boffset, add=True,
+                                 atomic=True)
+    assert_atomic_close(host(base), 2.0 * y_o)
+    # checksum: every in-image stack element lands exactly once (float64 sums agree to rounding)
+    ar = torch.arange(16, device=DEV)[None, :]
+    rows = (ar + 8 * idx_d[:, 1:2].long()) < H
+    cols = (ar + 8 * idx_d[:, 2:3].long()) < W
+    inside = (rows[:, :, None] & cols[:, None, :])[..., None]
+    assert abs(float(base.double().sum()) - 2.0 * float((stack.double() * inside).sum())) < 1e-3 * M
+
+
+def test_config5_many_small_images():
+    M = run_workload(workloads.config5())
+    assert M > 10000
