@@ -1,0 +1,360 @@
+#!/usr/bin/env python3
+"""Benchmark of the reduce_mask -> sparse_gather -> sparse_scatter path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--density 0.30] [--all-configs] [--no-cpu]
+
+A step is one pass of the path over the LiDAR-BEV-shaped workload (x = [1,800,800,128] fp32,
+27x27 blocks, stride 25, offset -1, max pooling, tol 0.5, `--density` of the 1024 blocks active):
+reduce_mask with the reference's host-visible count, sparse_gather with the fused transpose, and
+sparse_scatter_var in place (add=False, same geometry).  Inputs are resident in HBM before the timed
+region; three independent buffer sets (more than 1 GB in total) are rotated so the 256 MB Infinity
+Cache cannot serve one step's data to the next.  All calls go through the C ABI of libsbnet_amd.so
+with ctypes; PyTorch only owns the device buffers and the stream.
+
+One JSON line goes to stdout.  `value` is algorithmic bytes per step / wall time per step.  `ops`
+holds per-op device times (HIP events around batches of back-to-back launches on the launch stream),
+`roofline` the dominant kernel (the transposing gather) against the 8 TB/s HBM peak, `cpu_baseline`
+the single-threaded CPU oracle (the reference's CPU functors restated; the reference builds them
+without OpenMP) on the same workload on this machine's host cores.  Tables for the other
+configurations (`--all-configs`) go to stderr.
+
+Algorithmic bytes (B = bsize[0]*bsize[1]*C*4 per block, B_in its in-image part, M active blocks):
+  gather            M*(B_in + B) + 6*M      read x once per block element, write the stack
+  scatter add=False M*(B + B_in) + 6*M      read the stack, write the base
+  scatter add=True  M*(B + 2*B_in) + 6*M    read the stack, read-modify-write the base
+  reduce_mask       N*H*W*4 + 6*M + 4       every mask pixel once
+"""
+import argparse
+import ctypes
+import json
+import os
+import statistics
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--density", type=float, default=0.30)
+    ap.add_argument("--all-configs", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline (profiling runs)")
+    return ap.parse_args()
+
+
+I2 = ctypes.c_int32 * 2
+I64x4 = ctypes.c_int64 * 4
+
+
+def in_image_bytes(idx, bsize, bstride, boffset, H, W, C):
+    """Sum over blocks of the in-image part of the block, in bytes."""
+    h0 = boffset[0] + idx[:, 1].astype(np.int64) * bstride[0]
+    w0 = boffset[1] + idx[:, 2].astype(np.int64) * bstride[1]
+    rows = np.clip(np.minimum(h0 + bsize[0], H) - np.maximum(h0, 0), 0, None)
+    cols = np.clip(np.minimum(w0 + bsize[1], W) - np.maximum(w0, 0), 0, None)
+    return int((rows * cols).sum()) * C * 4
+
+
+class Path:
+    """Pre-allocated device buffers and raw C-ABI calls for one workload, `nsets` rotating copies."""
+
+    def __init__(self, wl, torch, lib, nsets=3, stack_fill=None):
+        self.wl, self.torch, self.lib = wl, torch, lib
+        dev = "cuda:0"
+        N, H, W, C = wl.shape
+        self.N, self.H, self.W, self.C = N, H, W, C
+        self.dims = I64x4(N, H, W, C)
+        self.bc, self.bs, self.bst, self.bo = I2(*wl.bcount), I2(*wl.bsize), I2(*wl.bstride), I2(*wl.boffset)
+        self.sbs, self.sbst, self.sbo = I2(*wl.s_bsize), I2(*wl.s_bstride), I2(*wl.s_boffset)
+        self.maxidx = N * wl.bcount[0] * wl.bcount[1]
+        self.nws = lib.sbnet_reduce_mask_workspace_bytes(N, self.bc, 2)
+        self.host_count = np.zeros(1, np.int32)
+        self.hc_ptr = self.host_count.ctypes.data_as(ctypes.POINTER(ctypes.c_int32))
+        self.stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        self.sets = []
+        if wl.indices is not None:
+            idx_host = np.ascontiguousarray(wl.indices, np.int16)
+            self.M = len(idx_host)
+        else:
+            from oracle import sbnet_oracle as orc  # only to size the buffers (M); not timed, not the product path
+            idx_host, cnt = orc.reduce_mask(wl.mask, wl.bcount, wl.bsize, wl.bstride, wl.boffset, wl.tol, wl.avgpool)
+            self.M = int(cnt[0])
+            idx_host = idx_host[:self.M]
+        self.idx_host = idx_host
+        R, S = wl.bsize
+        sR, sS = wl.s_bsize
+        for i in range(nsets):
+            s = {}
+            if wl.mask is not None:
+                s["mask"] = torch.from_numpy(wl.mask).to(dev)
+                s["idx"] = torch.zeros((self.maxidx, 3), dtype=torch.int16, device=dev)
+                s["idx"][:self.M] = torch.from_numpy(idx_host).to(dev)
+            else:
+                s["mask"] = None
+                s["idx"] = torch.from_numpy(idx_host).to(dev)
+            s["ws"] = torch.empty(max(self.nws, 16), dtype=torch.uint8, device=dev)
+            s["dcount"] = torch.zeros(1, dtype=torch.int32, device=dev)
+            if wl.x is not None:
+                s["x"] = torch.from_numpy(wl.x).to(dev)
+                s["stack"] = torch.empty((self.M, C, R, S) if wl.transpose else (self.M, R, S, C),
+                                         dtype=torch.float32, device=dev)
+            else:
+                s["x"] = None
+            shape = (self.M, C, sR, sS) if wl.transpose else (self.M, sR, sS, C)
+            if (sR, sS) == (R, S) and wl.x is not None:
+                s["sstack"] = s["stack"]
+            else:
+                g = torch.Generator(device=dev).manual_seed(4000 + i)
+                s["sstack"] = torch.rand(shape, generator=g, device=dev) * 2.0 - 1.0
+            s["base"] = torch.zeros((N, H, W, C), dtype=torch.float32, device=dev) if wl.x is None or not wl.s_var \
+                else s["x"]
+            if not wl.s_var:
+                s["out"] = torch.empty((N, H, W, C), dtype=torch.float32, device=dev)
+            self.sets.append(s)
+        torch.cuda.synchronize()
+        B = R * S * C * 4
+        sB = sR * sS * C * 4
+        bin_g = in_image_bytes(idx_host, wl.bsize, wl.bstride, wl.boffset, H, W, C)
+        bin_s = in_image_bytes(idx_host, wl.s_bsize, wl.s_bstride, wl.s_boffset, H, W, C)
+        M = self.M
+        self.bytes = {
+            "reduce_mask": N * H * W * 4 + 6 * M + 4,
+            "gather": bin_g + M * B + 6 * M,
+            "scatter": M * sB + (2 if wl.s_add else 1) * bin_s + 6 * M + (0 if wl.s_var else 2 * N * H * W * C * 4),
+        }
+
+    def check(self, rc):
+        if rc != 0:
+            raise RuntimeError("sbnet call failed: %s (hip %d)" % (self.lib.sbnet_status_string(rc).decode(),
+                                                                    self.lib.sbnet_last_hip_error()))
+
+    def reduce(self, i, sync=True):
+        s, wl = self.sets[i], self.wl
+        self.check(self.lib.sbnet_reduce_mask(s["mask"].data_ptr(), self.N, self.H, self.W, self.bc, 2, self.bs, 2,
+                                              self.bst, 2, self.bo, 2, wl.tol, int(wl.avgpool), s["idx"].data_ptr(),
+                                              self.hc_ptr if sync else None, s["dcount"].data_ptr(),
+                                              s["ws"].data_ptr(), self.nws, self.stream))
+        return int(self.host_count[0]) if sync else self.M
+
+    def gather(self, i, M):
+        s, wl = self.sets[i], self.wl
+        self.check(self.lib.sbnet_sparse_gather(s["x"].data_ptr(), self.dims, 4, M, s["idx"].data_ptr(), self.bs, 2,
+                                                self.bst, 2, self.bo, 2, int(wl.transpose), s["stack"].data_ptr(),
+                                                self.stream))
+
+    def scatter(self, i, M):
+        s, wl = self.sets[i], self.wl
+        if wl.s_var:
+            self.check(self.lib.sbnet_sparse_scatter_var(s["sstack"].data_ptr(), M, s["idx"].data_ptr(),
+                                                         s["base"].data_ptr(), self.dims, 4, self.sbs, 2, self.sbst, 2,
+                                                         self.sbo, 2, int(wl.s_add), int(wl.s_atomic),
+                                                         int(wl.transpose), self.stream))
+        else:
+            self.check(self.lib.sbnet_sparse_scatter(s["sstack"].data_ptr(), M, s["idx"].data_ptr(),
+                                                     s["base"].data_ptr(), self.dims, 4, self.sbs, 2, self.sbst, 2,
+                                                     self.sbo, 2, int(wl.s_add), int(wl.s_atomic), int(wl.transpose),
+                                                     s["out"].data_ptr(), self.stream))
+
+    def step(self, i):
+        M = self.reduce(i) if self.wl.mask is not None else self.M
+        if self.wl.x is not None:
+            self.gather(i, M)
+        self.scatter(i, M)
+        return M
+
+    def time_op(self, fn, batches=7, reps=12):
+        """Median device time per launch: HIP events around `reps` back-to-back launches on the stream
+        the kernels run on (torch's current stream), rotating over the buffer sets."""
+        torch = self.torch
+        n = len(self.sets)
+        for i in range(n):
+            fn(i)
+        torch.cuda.synchronize()
+        out = []
+        for b in range(batches):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for r in range(reps):
+                fn((b * reps + r) % n)
+            e1.record()
+            e1.synchronize()
+            out.append(e0.elapsed_time(e1) * 1e3 / reps)
+        return statistics.median(out)
+
+    def op_table(self):
+        ops = {}
+        if self.wl.mask is not None:
+            ops["reduce_mask"] = self.time_op(lambda i: self.reduce(i, sync=False))
+        if self.wl.x is not None:
+            ops["gather"] = self.time_op(lambda i: self.gather(i, self.M))
+        ops["scatter"] = self.time_op(lambda i: self.scatter(i, self.M))
+        table = {}
+        for k, us in ops.items():
+            gbs = self.bytes[k] / us * 1e-3
+            table[k] = {"us": round(us, 2), "bytes": self.bytes[k], "GBps": round(gbs, 1),
+                        "frac_of_8TBps": round(gbs / HBM_PEAK_GBS, 4)}
+        return table
+
+
+def cpu_baseline(wl, M, idx_host, nbytes, budget_s=12.0):
+    """Times the CPU oracle's gather + scatter (single thread: the reference's Makefile has no -fopenmp)
+    on the same workload, repeating until about `budget_s` seconds have been spent."""
+    from oracle import sbnet_oracle as orc
+    lib = orc.lib()
+    x = wl.x
+    N, H, W, C = wl.shape
+    R, S = wl.bsize
+    stack = np.empty((M, C, R, S) if wl.transpose else (M, R, S, C), np.float32)
+    base = x.copy()
+    f32p = ctypes.POINTER(ctypes.c_float)
+    i16p = ctypes.POINTER(ctypes.c_int16)
+    idx = np.ascontiguousarray(idx_host, np.int16)
+
+    def run(omp):
+        g = lib.oracle_sparse_gather_omp if omp else lib.oracle_sparse_gather
+        sc = lib.oracle_sparse_scatter_omp if omp else lib.oracle_sparse_scatter
+        t0 = time.perf_counter()
+        g(x.ctypes.data_as(f32p), N, H, W, C, stack.ctypes.data_as(f32p), wl.boffset[0], wl.boffset[1], R, S,
+          wl.bstride[0], wl.bstride[1], M, idx.ctypes.data_as(i16p), int(wl.transpose))
+        sc(stack.ctypes.data_as(f32p), N, H, W, C, base.ctypes.data_as(f32p), wl.s_boffset[0], wl.s_boffset[1],
+           wl.s_bsize[0], wl.s_bsize[1], wl.s_bstride[0], wl.s_bstride[1], M, idx.ctypes.data_as(i16p), int(wl.s_add),
+           int(wl.transpose), 0)
+        return time.perf_counter() - t0
+
+    run(False)
+    times, spent = [], 0.0
+    while spent < budget_s * 0.7 and len(times) < 40:
+        t = run(False)
+        times.append(t)
+        spent += t
+    t1 = statistics.median(times)
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    omp_threads = int(os.environ.get("OMP_NUM_THREADS", cores))
+    run(True)
+    times_omp, spent = [], 0.0
+    while spent < budget_s * 0.3 and len(times_omp) < 40:
+        t = run(True)
+        times_omp.append(t)
+        spent += t
+    tm = statistics.median(times_omp)
+    sample = "%s gather(transpose)+scatter_var, full workload (M=%d blocks), median of %d runs" % (wl.name, M, len(times))
+    return ({"value": round(nbytes / t1 * 1e-9, 3), "unit": "GB/s", "cores": 1, "kind": "port", "sample": sample,
+             "ms_per_pass": round(t1 * 1e3, 2)},
+            {"value": round(nbytes / tm * 1e-9, 3), "unit": "GB/s", "cores": omp_threads, "kind": "port",
+             "sample": sample.replace("median of %d" % len(times), "median of %d" % len(times_omp)) + ", OpenMP over blocks",
+             "ms_per_pass": round(tm * 1e3, 2)})
+
+
+def read_measured_traffic(name):
+    """HBM bytes per launch measured with rocprofv3 --pmc, if a summary under profiles/ records them as
+    lines `fetch_bytes_per_launch=<int>` and `write_bytes_per_launch=<int>`."""
+    p = os.path.join(ROOT, "profiles", name)
+    if not os.path.exists(p):
+        return None
+    vals = {}
+    for line in open(p):
+        for key in ("fetch_bytes_per_launch", "write_bytes_per_launch"):
+            if line.strip().startswith(key + "="):
+                vals[key] = int(float(line.split("=", 1)[1].split()[0]))
+    if len(vals) == 2:
+        return vals["fetch_bytes_per_launch"] + vals["write_bytes_per_launch"]
+    return None
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this path is measured on one GPU only (one MI355X per box); --gpus %d is not supported. "
+              "Sharding is by image (n) with no exchange; see DESIGN.md." % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    from sbnet_amd import _lib, workloads
+    lib = _lib.load()
+    torch.cuda.set_device(0)
+
+    wl = workloads.config3(args.density)
+    path = Path(wl, torch, lib, nsets=3)
+    nsets = len(path.sets)
+    for i in range(args.warmup):
+        path.step(i % nsets)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        M = path.step(i % nsets)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    assert M == path.M, "active block count changed between runs"
+    ms_per_step = wall / args.steps * 1e3
+    step_bytes = sum(path.bytes.values())
+    value = step_bytes / (ms_per_step * 1e-3) * 1e-9
+
+    ops = path.op_table()
+    g = ops["gather"]
+    roofline = {"bound": "hbm", "kernel": "k_gather_planar<4> (sparse_gather, transpose=True)",
+                "achieved": g["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(g["GBps"] / HBM_PEAK_GBS, 4), "us_per_launch": g["us"],
+                "algorithmic_bytes_per_launch": g["bytes"],
+                "traffic": read_measured_traffic("gather_planar_C3_pmc.txt")}
+    out = {
+        "metric": "achieved HBM GB/s over reduce_mask+sparse_gather+sparse_scatter_var (algorithmic bytes / wall time per step)",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "C3 LiDAR-BEV x=[1,800,800,128] fp32, bsize 27 bstride 25 boffset -1, max-pool tol 0.5, "
+                               "%d%% of 1024 blocks active (M=%d), gather transpose=True, scatter_var add=False in place"
+                               % (round(args.density * 100), path.M),
+                   "buffer_sets": nsets, "bytes_per_step": step_bytes},
+        "ops": ops, "roofline": roofline,
+    }
+    if not args.no_cpu:
+        nb = path.bytes["gather"] + path.bytes["scatter"]
+        one, omp = cpu_baseline(wl, path.M, path.idx_host, nb)
+        out["cpu_baseline"] = one
+        out["cpu_baseline_openmp"] = omp
+        gpu_gs = nb / ((ops["gather"]["us"] + ops["scatter"]["us"]) * 1e-6) * 1e-9
+        out["gather_plus_scatter_GBps"] = round(gpu_gs, 1)
+    print(json.dumps(out))
+    sys.stdout.flush()
+
+    if args.all_configs:
+        del path
+        torch.cuda.empty_cache()
+        rows = []
+        gens = [("C1", workloads.config1, {}), ("C2", workloads.config2, {}),
+                ("C3@5%", workloads.config3, {"density": 0.05}), ("C3@15%", workloads.config3, {"density": 0.15}),
+                ("C3@30%", workloads.config3, {"density": 0.30}), ("C4", workloads.config4, {}),
+                ("C5", workloads.config5, {})]
+        for name, gen, kw in gens:
+            w = gen(**kw)
+            p = Path(w, torch, lib, nsets=2 if name == "C4" else 3)
+            n = len(p.sets)
+            for i in range(5):
+                p.step(i % n)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            K = 50
+            for i in range(K):
+                p.step(i % n)
+            torch.cuda.synchronize()
+            e2e = (time.perf_counter() - t0) / K * 1e6
+            row = {"config": name, "M": p.M, "end_to_end_us": round(e2e, 1), "ops": p.op_table()}
+            rows.append(row)
+            print(json.dumps(row), file=sys.stderr)
+            del p
+            torch.cuda.empty_cache()
+
+
+if __name__ == "__main__":
+    main()

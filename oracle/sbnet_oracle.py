@@ -158,6 +158,9 @@ def sparse_scatter_var(x, bin_counts, active_block_indices, ybase, dynamic_bsize
 def sparse_scatter_raw(x, M, idx, y, bsize, bstride, boffset, add, transpose, omp=False):
     """Functor-level scatter into y in place (for timing: no validation, no copy)."""
     fn = lib().oracle_sparse_scatter_omp if omp else lib().oracle_sparse_scatter
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    idx = np.ascontiguousarray(idx, dtype=np.int16)
+    assert y.dtype == np.float32 and y.flags.c_contiguous
     N, H, W, C = y.shape
     fn(x.ctypes.data_as(_f32p), N, H, W, C, y.ctypes.data_as(_f32p), int(boffset[0]), int(boffset[1]),
        int(bsize[0]), int(bsize[1]), int(bstride[0]), int(bstride[1]), int(M),

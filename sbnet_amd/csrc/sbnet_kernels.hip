@@ -54,26 +54,33 @@ __device__ __forceinline__ uint32_t fdiv(uint32_t n, const FastDiv& f)
     return (t + ((n - t) >> f.sh1)) >> f.sh2;
 }
 
+// Native clang vectors (not HIP's float4 struct): they take the nontemporal builtins and arithmetic.
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef float f2 __attribute__((ext_vector_type(2)));
+
 template <int VEC> struct Vec;
-template <> struct Vec<4> { typedef float4 type; };
-template <> struct Vec<2> { typedef float2 type; };
+template <> struct Vec<4> { typedef f4 type; };
+template <> struct Vec<2> { typedef f2 type; };
 template <> struct Vec<1> { typedef float type; };
 
 template <int VEC> __device__ __forceinline__ typename Vec<VEC>::type vzero();
-template <> __device__ __forceinline__ float4 vzero<4>() { return make_float4(0.f, 0.f, 0.f, 0.f); }
-template <> __device__ __forceinline__ float2 vzero<2>() { return make_float2(0.f, 0.f); }
+template <> __device__ __forceinline__ f4 vzero<4>() { return (f4)(0.f); }
+template <> __device__ __forceinline__ f2 vzero<2>() { return (f2)(0.f); }
 template <> __device__ __forceinline__ float vzero<1>() { return 0.f; }
 
-__device__ __forceinline__ float vget(const float4& v, int k) { return k == 0 ? v.x : k == 1 ? v.y : k == 2 ? v.z : v.w; }
-__device__ __forceinline__ float vget(const float2& v, int k) { return k == 0 ? v.x : v.y; }
+__device__ __forceinline__ float vget(const f4& v, int k) { return k == 0 ? v.x : k == 1 ? v.y : k == 2 ? v.z : v.w; }
+__device__ __forceinline__ float vget(const f2& v, int k) { return k == 0 ? v.x : v.y; }
 __device__ __forceinline__ float vget(const float& v, int) { return v; }
-__device__ __forceinline__ void vset(float4& v, int k, float f) { if (k == 0) v.x = f; else if (k == 1) v.y = f; else if (k == 2) v.z = f; else v.w = f; }
-__device__ __forceinline__ void vset(float2& v, int k, float f) { if (k == 0) v.x = f; else v.y = f; }
+__device__ __forceinline__ void vset(f4& v, int k, float f) { if (k == 0) v.x = f; else if (k == 1) v.y = f; else if (k == 2) v.z = f; else v.w = f; }
+__device__ __forceinline__ void vset(f2& v, int k, float f) { if (k == 0) v.x = f; else v.y = f; }
 __device__ __forceinline__ void vset(float& v, int, float f) { v = f; }
 
-__device__ __forceinline__ float4 vadd(const float4& a, const float4& b) { return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w); }
-__device__ __forceinline__ float2 vadd(const float2& a, const float2& b) { return make_float2(a.x + b.x, a.y + b.y); }
-__device__ __forceinline__ float vadd(const float& a, const float& b) { return a + b; }
+template <typename T> __device__ __forceinline__ T vadd(const T& a, const T& b) { return a + b; }
+
+// Streaming accesses: every byte of x, of the block stack and of the base tensor is touched once per
+// op, so loads and stores carry the nontemporal hint (measured: a plain dwordx4 copy gains ~10 %).
+template <typename T> __device__ __forceinline__ T ld_stream(const T* p) { return __builtin_nontemporal_load(p); }
+template <typename T> __device__ __forceinline__ void st_stream(T* p, const T& v) { __builtin_nontemporal_store(v, p); }
 
 // Hardware fp32 atomic add (global_atomic_add_f32, no return value).
 __device__ __forceinline__ void atomic_add_f32(float* p, float v) { unsafeAtomicAdd(p, v); }
@@ -84,9 +91,9 @@ template <int VEC, int MODE>
 __device__ __forceinline__ void commit(typename Vec<VEC>::type* dst, const typename Vec<VEC>::type& v)
 {
     if (MODE == SCATTER_ASSIGN) {
-        *dst = v;
+        st_stream(dst, v);
     } else if (MODE == SCATTER_ADD) {
-        *dst = vadd(*dst, v);
+        st_stream(dst, vadd(ld_stream(dst), v));
     } else {
         float* d = reinterpret_cast<float*>(dst);
 #pragma unroll
@@ -111,6 +118,38 @@ __device__ __forceinline__ BlockOrigin load_origin(const int16_t* __restrict__ i
     return o;
 }
 
+// The same in two steps, for software pipelines: the loads are issued early and the arithmetic (which
+// is what makes a wave wait for them) happens where the origin is first needed.
+struct RawTriple {
+    uint32_t nbh;  // n in the low half, bh in the high half, exactly as loaded
+    int bw;
+};
+
+typedef uint32_t u32_a2 __attribute__((aligned(2)));
+
+__device__ __forceinline__ RawTriple load_triple(const int16_t* __restrict__ idx, uint32_t ib)
+{
+    const int16_t* t = idx + (size_t)ib * 3;
+    RawTriple r;
+    r.nbh = *reinterpret_cast<const u32_a2*>(t);
+    r.bw = t[2];
+    return r;
+}
+
+__device__ __forceinline__ BlockOrigin origin_of(const RawTriple& r, const Geom& g)
+{
+    BlockOrigin o;
+    o.n = (int)(int16_t)(r.nbh & 0xffffu);
+    o.h0 = g.oh + (int)(int16_t)(r.nbh >> 16) * g.U;
+    o.w0 = g.ow + r.bw * g.V;
+    o.valid = (unsigned)o.n < (unsigned)g.N;
+    return o;
+}
+
+// Sixteen zero bytes in device memory: where a pipelined load has nothing to fetch (a pixel outside
+// the image, a lane past the end of a tile) it reads these instead of branching around the load.
+__device__ const float g_zero16[4] __attribute__((aligned(16))) = {0.f, 0.f, 0.f, 0.f};
+
 // ---------------------------------------------------------------------------------------------
 // NHWC block stack <-> NHWC tensor: row-segment copies
 // ---------------------------------------------------------------------------------------------
@@ -119,7 +158,7 @@ __device__ __forceinline__ BlockOrigin load_origin(const int16_t* __restrict__ i
 // the tensor is R row segments of the same length (the in-range part of it).  One wave handles
 // one "unit": CHUNK = 64*UNR consecutive vectors of one block; four units per workgroup.
 
-constexpr int NHWC_UNR = 8;
+constexpr int NHWC_UNR = 4;  // 4 KB per wave, 16 KB per workgroup (see COPY_UNR)
 constexpr int NHWC_CHUNK = 64 * NHWC_UNR;
 
 struct NhwcArgs {
@@ -163,14 +202,14 @@ __global__ __launch_bounds__(256) void k_gather_nhwc(const float* __restrict__ x
             const int hh = o.h0 + (int)r;
             if (o.valid && (unsigned)hh < (unsigned)a.g.H && j >= lo && j < hi) {
                 const int64_t src = (((int64_t)o.n * a.g.H + hh) * a.g.W + o.w0) * CV + j;
-                v[u] = xv[src];
+                v[u] = ld_stream(xv + src);
             }
         }
     }
 #pragma unroll
     for (int u = 0; u < NHWC_UNR; ++u) {
         const uint32_t e = e0 + u * 64;
-        if (e < a.blockV) yb[e] = v[u];
+        if (e < a.blockV) st_stream(yb + e, v[u]);
     }
 }
 
@@ -208,7 +247,7 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
             const int hh = o.h0 + (int)r;
             if ((unsigned)hh < (unsigned)a.g.H && j >= lo && j < hi) {
                 dst[u] = (((int64_t)o.n * a.g.H + hh) * a.g.W + o.w0) * CV + j;
-                v[u] = xb[e];
+                v[u] = ld_stream(xb + e);
             }
         }
     }
@@ -216,10 +255,10 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
         vec cur[NHWC_UNR];
 #pragma unroll
         for (int u = 0; u < NHWC_UNR; ++u)
-            if (dst[u] >= 0) cur[u] = yv[dst[u]];
+            if (dst[u] >= 0) cur[u] = ld_stream(yv + dst[u]);
 #pragma unroll
         for (int u = 0; u < NHWC_UNR; ++u)
-            if (dst[u] >= 0) yv[dst[u]] = vadd(cur[u], v[u]);
+            if (dst[u] >= 0) st_stream(yv + dst[u], vadd(cur[u], v[u]));
     } else {
 #pragma unroll
         for (int u = 0; u < NHWC_UNR; ++u)
@@ -231,78 +270,134 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
 // planar block stack [blocks, C, R, S] <-> NHWC tensor: LDS-staged transpose
 // ---------------------------------------------------------------------------------------------
 //
-// One workgroup moves one tile: Ct channels x Pn pixels of one block, where pixels are numbered
-// p = r*S + s inside the block.  LDS holds the tile as [Ct][Pp] floats (row pitch Pp >= P, chosen
-// so the transposing accesses spread over the banks).  On the NHWC side a lane moves VEC channels
-// of one pixel (lanes of a wave cover Ct/VEC consecutive vectors of a pixel, then the next pixel);
-// on the planar side a wave moves one channel row of the tile, a contiguous run of Pn floats.
+// A tile is Ct channels x Pn pixels of one block, pixels numbered p = r*S + s inside the block.
+// On the NHWC side a lane moves VEC channels of one pixel (the lanes of a wave cover the Ct/VEC
+// vectors of a pixel, then the next pixel).  On the planar side row c of the tile is a contiguous
+// run of Pn floats that starts at whatever 4-byte alignment (c*R*S + p0) lands on (27x27 planes hold
+// 729 floats).  Runs move as dwordx4 "slots" of 4 consecutive floats from the start of the run, so
+// most of these accesses are not 16-byte aligned; gfx950 executes misaligned global dwordx4 accesses
+// at the speed of aligned ones (measured with a plain copy), which makes an aligned-body / scalar-
+// head-and-tail split unnecessary.  Only the last slot of a run can be partial.
 //
-// Workgroup ids are remapped so that the tiles of one block (its channel chunks and pixel splits)
-// run on the same XCD: hardware hands consecutive workgroup ids to the 8 XCDs round-robin, and
-// sibling tiles share cache lines (the 2 halves of a 128-byte line when Ct*4 = 64, the ragged
-// ends of planar runs), which only merge in an L2 they have in common.
+// Workgroups are persistent: each takes a contiguous range of tiles and software-pipelines them.
+// The global loads of tile i+1 are issued into registers before the stores of tile i leave LDS, so
+// a workgroup keeps reads and writes in flight at the same time instead of alternating between a
+// load phase and a store phase.  To keep that pipeline free of control flow around loads (which
+// would force the compiler to wait for each load where the branches join), every load is issued
+// unconditionally from an address that is always valid, and a bit mask remembers which registers
+// hold real data.  Tiles are ordered (block, channel chunk, pixel split) with the pixel split
+// fastest: the splits of one channel chunk continue each other's planar runs, and a workgroup that
+// owns them back to back lets the 128-byte lines shared at the seams merge in its XCD's L2.
+//
+// LDS layout: tile row c at c*Pp floats, Pp a multiple of 32, pixel e at column e.  Columns are
+// XOR-swizzled in units of 4 floats by ((c >> 2) & 7): the planar side still sees aligned groups of
+// 4 floats (ds_read_b128 / ds_write_b128), and the transposing NHWC side, where 32 lanes touch 4
+// consecutive pixels of 8 different channel groups at once, hits 32 distinct banks (LDS has 32
+// four-byte banks; a padded, unswizzled layout lost 58 % of its LDS cycles to bank conflicts).
+
+constexpr int TILE_LD = 8;  // vectors (NHWC side) or slots (planar side) held in registers per thread
+
+typedef f4 f4u __attribute__((aligned(4)));  // dwordx4 access at 4-byte alignment
 
 struct TileArgs {
     Geom g;
-    int Ct;         // channels per tile; Ct/VEC is a power of two
-    int lppLog;     // log2(Ct/VEC): lanes per pixel on the NHWC side
-    int P;          // pixels per tile (the last split of a block may hold fewer)
-    int Pp;         // LDS row pitch, floats
-    int psplit;     // pixel splits per block
-    int cchunks;    // channel chunks per block
-    uint32_t tpb;   // tiles per block = psplit * cchunks
-    uint32_t total; // numActive * tpb
-    uint32_t perXcd;  // ceil(total / 8); grid = 8 * perXcd
-    FastDiv dTpb, dCch, dS;
+    int Ct;             // channels per tile; Ct/VEC is a power of two
+    int lppLog;         // log2(Ct/VEC): lanes per pixel on the NHWC side
+    int P;              // pixels per tile (the last split of a block may hold fewer)
+    int Pp;             // LDS row pitch in floats, multiple of 32, >= P
+    int psplit;         // pixel splits per block
+    int cchunks;        // channel chunks per block
+    uint32_t tpb;       // tiles per block = psplit * cchunks
+    uint32_t total;     // numActive * tpb
+    uint32_t tilesPerWg;
+    uint32_t vpr;       // slots per planar row: (P + 3) / 4
+    FastDiv dTpb, dPs, dS, dVpr;
 };
-
-constexpr int TILE_UNR = 4;
 
 struct TileId {
     uint32_t ib;
     int c0, ctEff, p0, Pn;
 };
 
-__device__ __forceinline__ bool tile_of_workgroup(const TileArgs& a, TileId& t)
+__device__ __forceinline__ void decode_tile(const TileArgs& a, uint32_t id, TileId& t)
 {
-    const uint32_t bid = blockIdx.x;
-    const uint32_t id = (bid & 7u) * a.perXcd + (bid >> 3);
-    if (id >= a.total) return false;
     t.ib = fdiv(id, a.dTpb);
     const uint32_t rem = id - t.ib * a.tpb;
-    const uint32_t pc = fdiv(rem, a.dCch);
-    const uint32_t cc = rem - pc * a.cchunks;
+    const uint32_t cc = fdiv(rem, a.dPs);
+    const uint32_t pc = rem - cc * (uint32_t)a.psplit;
     t.c0 = (int)cc * a.Ct;
     t.ctEff = min(a.Ct, a.g.C - t.c0);
     t.p0 = (int)pc * a.P;
     t.Pn = min(a.P, a.g.R * a.g.S - t.p0);
-    return true;
 }
 
-// Copies one planar run (n floats) between LDS and global memory with an aligned dwordx4 body.
-// TO_GLOBAL: LDS -> global, else global -> LDS.  Called by one full wave.
-template <bool TO_GLOBAL>
-__device__ __forceinline__ void planar_run(float* __restrict__ gptr, float* __restrict__ lptr, int n, uint32_t lane)
+__device__ __forceinline__ uint32_t lds_swz(uint32_t c) { return ((c >> 2) & 7u) << 2; }
+
+// NHWC side, global -> registers.  Vector i = u*nthr + tid of the tile is pixel i >> lppLog, channel
+// vector i & (lpp - 1).  Pixels outside the image read as zero (sparse_gather.cc:80-82).
+template <int VEC>
+__device__ __forceinline__ void nhwc_load_tile(const typename Vec<VEC>::type* __restrict__ xv, const TileArgs& a,
+                                               const TileId& t, const BlockOrigin& o, uint32_t tid, uint32_t nthr,
+                                               typename Vec<VEC>::type (&v)[TILE_LD])
 {
-    const int mis = (int)((reinterpret_cast<uintptr_t>(gptr) >> 2) & 3);
-    const int head = min((4 - mis) & 3, n);
-    if ((int)lane < head) {
-        if (TO_GLOBAL) gptr[lane] = lptr[lane]; else lptr[lane] = gptr[lane];
+    typedef typename Vec<VEC>::type vec;
+    const uint32_t lppMask = (1u << a.lppLog) - 1u;
+    const uint32_t items = (uint32_t)t.Pn << a.lppLog;
+    const int CV = a.g.C / VEC;
+    // byte distance from x to the zero buffer: selecting an offset instead of a pointer keeps every
+    // access a global_load from one base
+    const int64_t zoff = reinterpret_cast<const char*>(g_zero16) - reinterpret_cast<const char*>(xv);
+#pragma unroll
+    for (int u = 0; u < TILE_LD; ++u) {
+        const uint32_t i = u * nthr + tid;
+        const uint32_t pl = i >> a.lppLog, cl = i & lppMask;
+        const uint32_t p = (uint32_t)t.p0 + pl;
+        const uint32_t r = fdiv(p, a.dS);
+        const int hh = o.h0 + (int)r, ww = o.w0 + (int)(p - r * a.g.S);
+        const int c = t.c0 + (int)cl * VEC;
+        const bool ok = i < items && o.valid && (unsigned)hh < (unsigned)a.g.H && (unsigned)ww < (unsigned)a.g.W &&
+                        c < a.g.C;
+        const int64_t src = (((int64_t)o.n * a.g.H + hh) * a.g.W + ww) * CV + (c / VEC);
+        v[u] = *reinterpret_cast<const vec*>(reinterpret_cast<const char*>(xv) + (ok ? src * (int64_t)sizeof(vec) : zoff));
     }
-    const int nb = (n - head) >> 2;
-    for (int v = (int)lane; v < nb; v += 64) {
-        const int o = head + 4 * v;
-        if (TO_GLOBAL) {
-            float4 t = make_float4(lptr[o], lptr[o + 1], lptr[o + 2], lptr[o + 3]);
-            *reinterpret_cast<float4*>(gptr + o) = t;
+}
+
+// Planar side, LDS -> global: slot i of the tile is row i / vpr, floats [4v, 4v + 4) of its run.
+__device__ __forceinline__ void planar_store_tile(float* __restrict__ g0, int64_t RS, const float* __restrict__ lds,
+                                                  const TileArgs& a, const TileId& t, uint32_t tid, uint32_t nthr)
+{
+    const uint32_t items = (uint32_t)t.ctEff * a.vpr;
+    for (uint32_t i = tid; i < items; i += nthr) {
+        const uint32_t c = fdiv(i, a.dVpr);
+        const uint32_t v = i - c * a.vpr;
+        const int e0 = 4 * (int)v;
+        if (e0 >= t.Pn) continue;
+        const f4 q = *reinterpret_cast<const f4*>(lds + c * a.Pp + ((4u * v) ^ lds_swz(c)));
+        float* __restrict__ dst = g0 + (int64_t)c * RS + e0;
+        if (e0 + 4 <= t.Pn) {
+            __builtin_nontemporal_store(q, reinterpret_cast<f4u*>(dst));
         } else {
-            float4 t = *reinterpret_cast<const float4*>(gptr + o);
-            lptr[o] = t.x; lptr[o + 1] = t.y; lptr[o + 2] = t.z; lptr[o + 3] = t.w;
+            dst[0] = q.x;
+            if (e0 + 1 < t.Pn) dst[1] = q.y;
+            if (e0 + 2 < t.Pn) dst[2] = q.z;
         }
     }
-    const int t0 = head + 4 * nb;
-    if ((int)lane < n - t0) {
-        if (TO_GLOBAL) gptr[t0 + lane] = lptr[t0 + lane]; else lptr[t0 + lane] = gptr[t0 + lane];
+}
+
+// Planar side, global -> registers.  The last slot of a run, when partial, is read as the last 4
+// floats of the run instead (overlapping its neighbour), so no load ever leaves the run and no loaded
+// value needs fixing up before it goes to LDS.  Needs Pn >= 4.
+__device__ __forceinline__ void planar_load_tile(const float* __restrict__ g0, int64_t RS, const TileArgs& a,
+                                                 const TileId& t, uint32_t tid, uint32_t nthr, f4 (&val)[TILE_LD])
+{
+    const uint32_t items = (uint32_t)t.ctEff * a.vpr;
+#pragma unroll
+    for (int u = 0; u < TILE_LD; ++u) {
+        const uint32_t i = u * nthr + tid;
+        const uint32_t c = fdiv(i, a.dVpr);
+        const int e0 = min(4 * (int)(i - c * a.vpr), t.Pn - 4);
+        const bool ok = i < items && e0 >= 0;
+        val[u] = *reinterpret_cast<const f4u*>(ok ? g0 + (int64_t)c * RS + e0 : g0);
     }
 }
 
@@ -312,49 +407,65 @@ __global__ __launch_bounds__(256) void k_gather_planar(const float* __restrict__
                                                        const int16_t* __restrict__ idx, TileArgs a)
 {
     typedef typename Vec<VEC>::type vec;
-    extern __shared__ float lds[];
-    TileId t;
-    if (!tile_of_workgroup(a, t)) return;
-    const BlockOrigin o = load_origin(idx, t.ib, a.g);
+    extern __shared__ __attribute__((aligned(16))) float lds[];
     const uint32_t tid = threadIdx.x, nthr = blockDim.x;
+    uint32_t tile = blockIdx.x * a.tilesPerWg;
+    const uint32_t tileEnd = min(a.total, tile + a.tilesPerWg);
+    if (tile >= tileEnd) return;
     const uint32_t lppMask = (1u << a.lppLog) - 1u;
-    const uint32_t items = (uint32_t)t.Pn << a.lppLog;
-    const vec* __restrict__ xv = reinterpret_cast<const vec*>(x);
-    const int CV = a.g.C / VEC;
-
-    for (uint32_t base = 0; base < items; base += nthr * TILE_UNR) {
-        vec v[TILE_UNR];
-#pragma unroll
-        for (int u = 0; u < TILE_UNR; ++u) {
-            const uint32_t i = base + u * nthr + tid;
-            v[u] = vzero<VEC>();
-            if (i < items) {
-                const uint32_t pl = i >> a.lppLog, cl = i & lppMask;
-                const uint32_t p = (uint32_t)t.p0 + pl;
-                const uint32_t r = fdiv(p, a.dS);
-                const int hh = o.h0 + (int)r, ww = o.w0 + (int)(p - r * a.g.S);
-                const int c = t.c0 + (int)cl * VEC;
-                if (o.valid && (unsigned)hh < (unsigned)a.g.H && (unsigned)ww < (unsigned)a.g.W && c < a.g.C)
-                    v[u] = xv[(((int64_t)o.n * a.g.H + hh) * a.g.W + ww) * CV + (c / VEC)];
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < TILE_UNR; ++u) {
-            const uint32_t i = base + u * nthr + tid;
-            if (i < items) {
-                const uint32_t pl = i >> a.lppLog, cl = i & lppMask;
-#pragma unroll
-                for (int k = 0; k < VEC; ++k) lds[(cl * VEC + k) * a.Pp + pl] = vget(v[u], k);
-            }
-        }
-    }
-    __syncthreads();
-
-    const uint32_t lane = tid & 63, wave = tid >> 6, nwaves = nthr >> 6;
     const int64_t RS = (int64_t)a.g.R * a.g.S;
-    for (int c = (int)wave; c < t.ctEff; c += (int)nwaves) {
-        float* dst = y + ((int64_t)t.ib * a.g.C + t.c0 + c) * RS + t.p0;
-        planar_run<true>(dst, lds + c * a.Pp, t.Pn, lane);
+    const vec* __restrict__ xv = reinterpret_cast<const vec*>(x);
+
+    // Pipeline state: `cur` is in registers (v) on its way to LDS, `nxt` is the tile whose loads are
+    // issued while `cur` is stored; block triples are fetched one tile further ahead so that no wave
+    // ever waits on an index load with nothing else in flight.
+    TileId cur, nxt;
+    decode_tile(a, tile, cur);
+    vec v[TILE_LD];
+    nhwc_load_tile<VEC>(xv, a, cur, load_origin(idx, cur.ib, a.g), tid, nthr, v);
+    bool more = tile + 1 < tileEnd;
+    nxt = cur;
+    RawTriple rawNext = {0u, 0};
+    if (more) {
+        decode_tile(a, tile + 1, nxt);
+        rawNext = load_triple(idx, nxt.ib);
+    }
+
+    for (;;) {
+        const uint32_t items = (uint32_t)cur.Pn << a.lppLog;
+#pragma unroll
+        for (int u = 0; u < TILE_LD; ++u) {
+            const uint32_t i = u * nthr + tid;
+            if (i < items) {
+                const uint32_t pl = i >> a.lppLog, cl = i & lppMask;
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    const uint32_t c = cl * VEC + k;
+                    lds[c * a.Pp + (pl ^ lds_swz(c))] = vget(v[u], k);
+                }
+            }
+        }
+        __syncthreads();
+        float* __restrict__ g0 = y + ((int64_t)cur.ib * a.g.C + cur.c0) * RS + cur.p0;
+        TileId nn = nxt;
+        RawTriple rawNn = rawNext;
+        const bool more2 = tile + 2 < tileEnd;
+        if (more) nhwc_load_tile<VEC>(xv, a, nxt, origin_of(rawNext, a.g), tid, nthr, v);
+        planar_store_tile(g0, RS, lds, a, cur, tid, nthr);
+        if (!more) break;
+        // The triple of the tile after next is fetched last: the wave makes it uniform at once, which
+        // waits for it, and memory operations retire in order - issued before the tile loads it would
+        // make every wave wait for those loads here instead of at the top of the loop.
+        if (more2) {
+            decode_tile(a, tile + 2, nn);
+            rawNn = load_triple(idx, nn.ib);
+        }
+        __syncthreads();
+        ++tile;
+        cur = nxt;
+        nxt = nn;
+        rawNext = rawNn;
+        more = more2;
     }
 }
 
@@ -364,59 +475,125 @@ __global__ __launch_bounds__(256) void k_scatter_planar(const float* __restrict_
                                                         const int16_t* __restrict__ idx, TileArgs a)
 {
     typedef typename Vec<VEC>::type vec;
-    extern __shared__ float lds[];
-    TileId t;
-    if (!tile_of_workgroup(a, t)) return;
-    const BlockOrigin o = load_origin(idx, t.ib, a.g);
-    if (!o.valid) return;
+    extern __shared__ __attribute__((aligned(16))) float lds[];
     const uint32_t tid = threadIdx.x, nthr = blockDim.x;
-    const uint32_t lane = tid & 63, wave = tid >> 6, nwaves = nthr >> 6;
-    const int64_t RS = (int64_t)a.g.R * a.g.S;
-
-    for (int c = (int)wave; c < t.ctEff; c += (int)nwaves) {
-        const float* src = x + ((int64_t)t.ib * a.g.C + t.c0 + c) * RS + t.p0;
-        planar_run<false>(const_cast<float*>(src), lds + c * a.Pp, t.Pn, lane);
-    }
-    __syncthreads();
-
+    uint32_t tile = blockIdx.x * a.tilesPerWg;
+    const uint32_t tileEnd = min(a.total, tile + a.tilesPerWg);
+    if (tile >= tileEnd) return;
     const uint32_t lppMask = (1u << a.lppLog) - 1u;
-    const uint32_t items = (uint32_t)t.Pn << a.lppLog;
+    const int64_t RS = (int64_t)a.g.R * a.g.S;
     vec* __restrict__ yv = reinterpret_cast<vec*>(y);
     const int CV = a.g.C / VEC;
 
-    for (uint32_t base = 0; base < items; base += nthr * TILE_UNR) {
-        vec v[TILE_UNR];
-        int64_t dst[TILE_UNR];
+    TileId cur;
+    decode_tile(a, tile, cur);
+    RawTriple raw = load_triple(idx, cur.ib);  // consumed after the planar loads below have landed
+    f4 val[TILE_LD];
+    planar_load_tile(x + ((int64_t)cur.ib * a.g.C + cur.c0) * RS + cur.p0, RS, a, cur, tid, nthr, val);
+
+    for (;;) {
+        const uint32_t slots = (uint32_t)cur.ctEff * a.vpr;
 #pragma unroll
-        for (int u = 0; u < TILE_UNR; ++u) {
-            const uint32_t i = base + u * nthr + tid;
-            dst[u] = -1;
-            v[u] = vzero<VEC>();
-            if (i < items) {
-                const uint32_t pl = i >> a.lppLog, cl = i & lppMask;
-                const uint32_t p = (uint32_t)t.p0 + pl;
-                const uint32_t r = fdiv(p, a.dS);
-                const int hh = o.h0 + (int)r, ww = o.w0 + (int)(p - r * a.g.S);
-                const int c = t.c0 + (int)cl * VEC;
-                if ((unsigned)hh < (unsigned)a.g.H && (unsigned)ww < (unsigned)a.g.W && c < a.g.C) {
-                    dst[u] = (((int64_t)o.n * a.g.H + hh) * a.g.W + ww) * CV + (c / VEC);
-#pragma unroll
-                    for (int k = 0; k < VEC; ++k) vset(v[u], k, lds[(cl * VEC + k) * a.Pp + pl]);
+        for (int u = 0; u < TILE_LD; ++u) {
+            const uint32_t i = u * nthr + tid;
+            if (i < slots) {
+                const uint32_t c = fdiv(i, a.dVpr);
+                const uint32_t vs = i - c * a.vpr;
+                const int e0 = 4 * (int)vs;
+                float* __restrict__ row = lds + c * a.Pp;
+                if (e0 + 4 <= cur.Pn) {
+                    *reinterpret_cast<f4*>(row + ((uint32_t)e0 ^ lds_swz(c))) = val[u];
+                } else if (e0 < cur.Pn) {  // partial last slot: holds floats [Pn-4, Pn) of the run
+                    const uint32_t t0 = (uint32_t)(cur.Pn - 4);
+                    row[(t0 + 0) ^ lds_swz(c)] = val[u].x;
+                    row[(t0 + 1) ^ lds_swz(c)] = val[u].y;
+                    row[(t0 + 2) ^ lds_swz(c)] = val[u].z;
+                    row[(t0 + 3) ^ lds_swz(c)] = val[u].w;
                 }
             }
         }
-        if (MODE == SCATTER_ADD) {
-            vec cur[TILE_UNR];
+        __syncthreads();
+        const bool more = tile + 1 < tileEnd;
+        const TileId done = cur;
+        const BlockOrigin od = origin_of(raw, a.g);
+        if (more) {
+            decode_tile(a, tile + 1, cur);
+            planar_load_tile(x + ((int64_t)cur.ib * a.g.C + cur.c0) * RS + cur.p0, RS, a, cur, tid, nthr, val);
+        }
+        // NHWC side of the finished tile: LDS -> base tensor; pixels outside the image are dropped
+        // (sparse_gather.cc:121).
+        if (od.valid) {
+            const uint32_t items = (uint32_t)done.Pn << a.lppLog;
+            for (uint32_t base = 0; base < items; base += nthr * 4) {
+                vec w[4];
+                int64_t dst[4];
 #pragma unroll
-            for (int u = 0; u < TILE_UNR; ++u)
-                if (dst[u] >= 0) cur[u] = yv[dst[u]];
+                for (int u = 0; u < 4; ++u) {
+                    const uint32_t i = base + u * nthr + tid;
+                    dst[u] = -1;
+                    w[u] = vzero<VEC>();
+                    if (i < items) {
+                        const uint32_t pl = i >> a.lppLog, cl = i & lppMask;
+                        const uint32_t p = (uint32_t)done.p0 + pl;
+                        const uint32_t r = fdiv(p, a.dS);
+                        const int hh = od.h0 + (int)r, ww = od.w0 + (int)(p - r * a.g.S);
+                        const int cg = done.c0 + (int)cl * VEC;
+                        if ((unsigned)hh < (unsigned)a.g.H && (unsigned)ww < (unsigned)a.g.W && cg < a.g.C) {
+                            dst[u] = (((int64_t)od.n * a.g.H + hh) * a.g.W + ww) * CV + (cg / VEC);
 #pragma unroll
-            for (int u = 0; u < TILE_UNR; ++u)
-                if (dst[u] >= 0) yv[dst[u]] = vadd(cur[u], v[u]);
-        } else {
+                            for (int k = 0; k < VEC; ++k) {
+                                const uint32_t c = cl * VEC + k;
+                                vset(w[u], k, lds[c * a.Pp + (pl ^ lds_swz(c))]);
+                            }
+                        }
+                    }
+                }
+                if (MODE == SCATTER_ADD) {
+                    vec curv[4];
 #pragma unroll
-            for (int u = 0; u < TILE_UNR; ++u)
-                if (dst[u] >= 0) commit<VEC, MODE>(yv + dst[u], v[u]);
+                    for (int u = 0; u < 4; ++u)
+                        if (dst[u] >= 0) curv[u] = ld_stream(yv + dst[u]);
+#pragma unroll
+                    for (int u = 0; u < 4; ++u)
+                        if (dst[u] >= 0) st_stream(yv + dst[u], vadd(curv[u], w[u]));
+                } else {
+#pragma unroll
+                    for (int u = 0; u < 4; ++u)
+                        if (dst[u] >= 0) commit<VEC, MODE>(yv + dst[u], w[u]);
+                }
+            }
+        }
+        if (!more) break;
+        raw = load_triple(idx, cur.ib);  // after the stores, see k_gather_planar
+        __syncthreads();
+        ++tile;
+    }
+}
+
+// Fallback for block planes of fewer than 4 pixels (1x1, 1x2, 1x3 ... blocks), where a dwordx4 slot does
+// not fit into a planar run: one thread per stack element.  The channel index varies fastest across
+// threads, so the NHWC side stays coalesced.
+template <int MODE, bool GATHER>
+__global__ __launch_bounds__(256) void k_planar_small(const float* __restrict__ x, float* __restrict__ y,
+                                                      const int16_t* __restrict__ idx, Geom g, int64_t total)
+{
+    const int RS = g.R * g.S;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const int c = (int)(i % g.C);
+        const int p = (int)((i / g.C) % RS);
+        const int64_t ib = i / ((int64_t)g.C * RS);
+        const int r = p / g.S, s = p - r * g.S;
+        const BlockOrigin o = load_origin(idx, (uint32_t)ib, g);
+        const int hh = o.h0 + r, ww = o.w0 + s;
+        const bool in = o.valid && (unsigned)hh < (unsigned)g.H && (unsigned)ww < (unsigned)g.W;
+        const int64_t pix = (((int64_t)o.n * g.H + hh) * g.W + ww) * g.C + c;
+        const int64_t st = (ib * g.C + c) * RS + p;
+        if (GATHER) {
+            y[st] = in ? x[pix] : 0.f;
+        } else if (in) {
+            if (MODE == SCATTER_ASSIGN) y[pix] = x[st];
+            else if (MODE == SCATTER_ADD) y[pix] += x[st];
+            else atomic_add_f32(y + pix, x[st]);
         }
     }
 }
@@ -614,22 +791,22 @@ __global__ __launch_bounds__(256) void k_reduce_compact(const uint8_t* __restric
 // flat copy (CopyTensorFunctor, sparse_gather.cc:135-142 / sparse_gather.cu:268-276)
 // ---------------------------------------------------------------------------------------------
 
-constexpr int COPY_UNR = 8;
+constexpr int COPY_UNR = 4;  // 16 KB per workgroup; 32 KB per workgroup measured 30 % slower
 
-__global__ __launch_bounds__(256) void k_copy_v4(const float4* __restrict__ src, float4* __restrict__ dst, size_t n4)
+__global__ __launch_bounds__(256) void k_copy_v4(const f4* __restrict__ src, f4* __restrict__ dst, size_t n4)
 {
     const size_t base = (size_t)blockIdx.x * (256 * COPY_UNR) + threadIdx.x;
-    float4 v[COPY_UNR];
+    f4 v[COPY_UNR];
 #pragma unroll
     for (int u = 0; u < COPY_UNR; ++u) {
         const size_t i = base + (size_t)u * 256;
-        v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (i < n4) v[u] = src[i];
+        v[u] = (f4)(0.f);
+        if (i < n4) v[u] = ld_stream(src + i);
     }
 #pragma unroll
     for (int u = 0; u < COPY_UNR; ++u) {
         const size_t i = base + (size_t)u * 256;
-        if (i < n4) dst[i] = v[u];
+        if (i < n4) st_stream(dst + i, v[u]);
     }
 }
 
@@ -656,9 +833,9 @@ static uint32_t pow2_ceil(uint32_t v)
     return p;
 }
 
-// Optional overrides for experiments: SBNET_TUNE="ct=32,lds=49152,wg=256".
+// Optional overrides for experiments: SBNET_TUNE="ct=32,lds=32768,occ=4".
 struct Tune {
-    int ct = 0, ldsBytes = 0, wg = 0;
+    int ct = 0, ldsBytes = 0, wg = 0, occ = 0;
 };
 
 static Tune read_tune()
@@ -670,6 +847,7 @@ static Tune read_tune()
     if ((p = strstr(s, "ct="))) t.ct = atoi(p + 3);
     if ((p = strstr(s, "lds="))) t.ldsBytes = atoi(p + 4);
     if ((p = strstr(s, "wg="))) t.wg = atoi(p + 3);
+    if ((p = strstr(s, "occ="))) t.occ = atoi(p + 4);
     return t;
 }
 
@@ -755,8 +933,23 @@ static bool make_nhwc_args(const Geom& g, int numActive, int vec, NhwcArgs& a)
     return true;
 }
 
-// Chooses the LDS tile of the planar kernels.
-static bool make_tile_args(const Geom& g, int numActive, int vec, TileArgs& a, int& threads, size_t& ldsBytes)
+// Compute units of the current device (cached per device index; read-only after the first query).
+static int device_cu_count()
+{
+    static int cus[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cus[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cus[dev] = n;
+    }
+    return cus[dev];
+}
+
+// Chooses the tile, the workgroup size and the persistent grid of the planar kernels.
+static bool make_tile_args(const Geom& g, int numActive, int vec, TileArgs& a, int& threads, size_t& ldsBytes,
+                           unsigned& grid)
 {
     static const Tune tune = read_tune();
     a.g = g;
@@ -764,40 +957,54 @@ static bool make_tile_args(const Geom& g, int numActive, int vec, TileArgs& a, i
     if (RS64 >= (1ll << 30)) return false;
     const int RS = (int)RS64;
     // channels per tile: 32 floats (one 128-byte line per pixel) unless C is smaller
-    int ctWant = tune.ct > 0 ? tune.ct : 32;
+    const int ctWant = tune.ct > 0 ? tune.ct : 32;
     int lpp = 1;
     while (lpp * 2 * vec <= ctWant && lpp * vec < g.C) lpp *= 2;
     a.Ct = lpp * vec;
     a.lppLog = ilog2_floor((uint32_t)lpp);
     a.cchunks = (g.C + a.Ct - 1) / a.Ct;
-    // pixels per tile: keep a tile within the LDS budget so several workgroups share a CU
-    const int budget = tune.ldsBytes > 0 ? tune.ldsBytes : 40 * 1024;
-    int maxP = budget / (a.Ct * 4) - 16;
-    if (maxP < 16) maxP = 16;
+    // Pixels per tile are bounded by the LDS budget and by the TILE_LD registers per thread that hold a
+    // tile in flight on either side.  The smallest workgroup that takes a whole block plane wins.
+    const int budget = tune.ldsBytes > 0 ? tune.ldsBytes : 32 * 1024;
+    int maxP = 0;
+    threads = 0;
+    for (int nthr = 64; nthr <= 256; nthr *= 2) {
+        const int pLds = (budget / (4 * a.Ct)) / 32 * 32;
+        const int pItems = TILE_LD * nthr / lpp;
+        const int pSlots = (TILE_LD * nthr / a.Ct) * 4 - 3;
+        maxP = pLds < pItems ? pLds : pItems;
+        if (pSlots < maxP) maxP = pSlots;
+        threads = nthr;
+        if (maxP >= RS) break;
+    }
+    if (tune.wg > 0 && tune.wg != threads) return false;  // experiments must pick a consistent size
+    if (maxP < 1) return false;
     a.psplit = (RS + maxP - 1) / maxP;
     a.P = (RS + a.psplit - 1) / a.psplit;
     a.psplit = (RS + a.P - 1) / a.P;
-    // pitch: vec*Pp == 64/lpp (mod 64) makes a wave's transposing LDS accesses hit 64 distinct banks
-    int Pp = a.P;
-    if (lpp * vec <= 64) {
-        const int want = (64 / lpp) % 64;
-        while ((vec * Pp) % 64 != want) ++Pp;
-    } else {
-        Pp |= 1;
-    }
-    a.Pp = Pp;
+    a.Pp = (a.P + 31) / 32 * 32;
+    a.vpr = (uint32_t)((a.P + 3) / 4);
     a.tpb = (uint32_t)(a.psplit * a.cchunks);
     const uint64_t total = (uint64_t)numActive * a.tpb;
-    if (total >= (1ull << 31) - 8) return false;
+    if (total >= (1ull << 31)) return false;
     a.total = (uint32_t)total;
-    a.perXcd = (a.total + 7) / 8;
     a.dTpb = make_fastdiv(a.tpb);
-    a.dCch = make_fastdiv((uint32_t)a.cchunks);
+    a.dPs = make_fastdiv((uint32_t)a.psplit);
     a.dS = make_fastdiv((uint32_t)g.S);
+    a.dVpr = make_fastdiv(a.vpr);
     ldsBytes = (size_t)a.Ct * a.Pp * sizeof(float);
-    const int elems = a.Ct * a.P;
-    threads = tune.wg > 0 ? tune.wg : (elems >= 4096 ? 256 : elems >= 1536 ? 128 : 64);
-    return ldsBytes <= 64 * 1024;
+    if (ldsBytes > 64 * 1024) return false;
+    // persistent grid: as many workgroups as the device holds at once (LDS, 2048 threads and 32 waves per CU)
+    int perCu = (int)((160 * 1024) / (ldsBytes + 512));
+    const int byThreads = 2048 / threads;
+    if (perCu > byThreads) perCu = byThreads;
+    if (tune.occ > 0 && perCu > tune.occ) perCu = tune.occ;
+    if (perCu < 1) perCu = 1;
+    const uint64_t slots = (uint64_t)device_cu_count() * perCu;
+    a.tilesPerWg = (uint32_t)((total + slots - 1) / slots);
+    if (a.tilesPerWg < 1) a.tilesPerWg = 1;
+    grid = (unsigned)((total + a.tilesPerWg - 1) / a.tilesPerWg);
+    return true;
 }
 
 template <int VEC>
@@ -812,8 +1019,16 @@ static void gather_dispatch(const float* x, float* y, const int16_t* idx, const 
         TileArgs a;
         int threads;
         size_t lds;
-        if (!make_tile_args(g, numActive, VEC, a, threads, lds)) { err = hipErrorInvalidValue; return; }
-        hipLaunchKernelGGL(k_gather_planar<VEC>, dim3(a.perXcd * 8), dim3(threads), lds, stream, x, y, idx, a);
+        unsigned grid;
+        if ((int64_t)g.R * g.S < 4) {
+            const int64_t total = (int64_t)numActive * g.C * g.R * g.S;
+            const int64_t wgs = (total + 255) / 256;
+            hipLaunchKernelGGL((k_planar_small<SCATTER_ASSIGN, true>), dim3((unsigned)(wgs > 65536 ? 65536 : wgs)),
+                               dim3(256), 0, stream, x, y, idx, g, total);
+            return;
+        }
+        if (!make_tile_args(g, numActive, VEC, a, threads, lds, grid)) { err = hipErrorInvalidValue; return; }
+        hipLaunchKernelGGL(k_gather_planar<VEC>, dim3(grid), dim3(threads), lds, stream, x, y, idx, a);
     }
 }
 
@@ -843,8 +1058,16 @@ static void scatter_dispatch(const float* x, float* y, const int16_t* idx, const
         TileArgs a;
         int threads;
         size_t lds;
-        if (!make_tile_args(g, numActive, VEC, a, threads, lds)) { err = hipErrorInvalidValue; return; }
-        hipLaunchKernelGGL((k_scatter_planar<VEC, MODE>), dim3(a.perXcd * 8), dim3(threads), lds, stream, x, y, idx, a);
+        unsigned grid;
+        if ((int64_t)g.R * g.S < 4) {
+            const int64_t total = (int64_t)numActive * g.C * g.R * g.S;
+            const int64_t wgs = (total + 255) / 256;
+            hipLaunchKernelGGL((k_planar_small<MODE, false>), dim3((unsigned)(wgs > 65536 ? 65536 : wgs)), dim3(256),
+                               0, stream, x, y, idx, g, total);
+            return;
+        }
+        if (!make_tile_args(g, numActive, VEC, a, threads, lds, grid)) { err = hipErrorInvalidValue; return; }
+        hipLaunchKernelGGL((k_scatter_planar<VEC, MODE>), dim3(grid), dim3(threads), lds, stream, x, y, idx, a);
     }
 }
 
@@ -879,7 +1102,7 @@ hipError_t launch_copy(float* dst, const float* src, size_t count, hipStream_t s
         if (n4) {
             const size_t per = 256 * COPY_UNR;
             hipLaunchKernelGGL(k_copy_v4, dim3((unsigned)((n4 + per - 1) / per)), dim3(256), 0, stream,
-                               reinterpret_cast<const float4*>(src), reinterpret_cast<float4*>(dst), n4);
+                               reinterpret_cast<const f4*>(src), reinterpret_cast<f4*>(dst), n4);
         }
         const size_t rem = count - n4 * 4;
         if (rem) hipLaunchKernelGGL(k_copy_scalar, dim3(1), dim3(256), 0, stream, src + n4 * 4, dst + n4 * 4, rem);

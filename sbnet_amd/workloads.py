@@ -136,7 +136,7 @@ def config4(seed=1004, shape=(2, 512, 512, 256)):
     N, H, W, C = shape
     bcount = [1 + (H - 1) // 8, 1 + (W - 1) // 8]
     cells = rng.random((N, bcount[0], bcount[1])) < 0.25
-    idx = np.argwhere(cells).astype(np.int16)
+    idx = np.ascontiguousarray(np.argwhere(cells), dtype=np.int16)  # argwhere returns a transposed view
     return _wl(name="C4", shape=list(shape), bsize=[16, 16], bstride=[8, 8], boffset=[0, 0], bcount=bcount, tol=0.5,
                avgpool=False, transpose=False, s_bsize=[16, 16], s_bstride=[8, 8], s_boffset=[0, 0], s_add=True,
                s_atomic=True, s_var=True, indices=idx)
