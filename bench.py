@@ -77,6 +77,7 @@ class Path:
         self.sbs, self.sbst, self.sbo = I2(*wl.s_bsize), I2(*wl.s_bstride), I2(*wl.s_boffset)
         self.maxidx = N * wl.bcount[0] * wl.bcount[1]
         self.nws = lib.sbnet_reduce_mask_workspace_bytes(N, self.bc, 2)
+        self.use_scatter_ws = True
         self.host_count = np.zeros(1, np.int32)
         self.hc_ptr = self.host_count.ctypes.data_as(ctypes.POINTER(ctypes.c_int32))
         self.stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
@@ -102,6 +103,9 @@ class Path:
                 s["mask"] = None
                 s["idx"] = torch.from_numpy(idx_host).to(dev)
             s["ws"] = torch.empty(max(self.nws, 16), dtype=torch.uint8, device=dev)
+            nsw = lib.sbnet_sparse_scatter_workspace_bytes(self.M, self.dims, 4, self.sbs, 2, self.sbst, 2, self.sbo, 2) \
+                if (wl.s_add and wl.s_atomic and not wl.transpose) else 0
+            s["sws"] = torch.empty(nsw, dtype=torch.uint8, device=dev) if nsw else None
             s["dcount"] = torch.zeros(1, dtype=torch.int32, device=dev)
             if wl.x is not None:
                 s["x"] = torch.from_numpy(wl.x).to(dev)
@@ -153,16 +157,18 @@ class Path:
 
     def scatter(self, i, M):
         s, wl = self.sets[i], self.wl
+        ws = s["sws"] if self.use_scatter_ws else None
+        wp, wn = (ws.data_ptr(), ws.numel()) if ws is not None else (None, 0)
         if wl.s_var:
             self.check(self.lib.sbnet_sparse_scatter_var(s["sstack"].data_ptr(), M, s["idx"].data_ptr(),
                                                          s["base"].data_ptr(), self.dims, 4, self.sbs, 2, self.sbst, 2,
                                                          self.sbo, 2, int(wl.s_add), int(wl.s_atomic),
-                                                         int(wl.transpose), self.stream))
+                                                         int(wl.transpose), wp, wn, self.stream))
         else:
             self.check(self.lib.sbnet_sparse_scatter(s["sstack"].data_ptr(), M, s["idx"].data_ptr(),
                                                      s["base"].data_ptr(), self.dims, 4, self.sbs, 2, self.sbst, 2,
                                                      self.sbo, 2, int(wl.s_add), int(wl.s_atomic), int(wl.transpose),
-                                                     s["out"].data_ptr(), self.stream))
+                                                     s["out"].data_ptr(), wp, wn, self.stream))
 
     def step(self, i):
         M = self.reduce(i) if self.wl.mask is not None else self.M

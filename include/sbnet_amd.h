@@ -150,6 +150,13 @@ int sbnet_sparse_gather_functor(const float* x, int N, int H, int W, int C, floa
  * sparse_scatter / sparse_scatter_var
  * ---------------------------------------------------------------------------------------- */
 
+/* Bytes of scratch that let an overlapping atomic scatter-add run without atomics (see workspace below);
+   0 when the method does not apply to this geometry. */
+size_t sbnet_sparse_scatter_workspace_bytes(int32_t num_active, const int64_t* ybase_dims, int ybase_rank,
+                                            const int32_t* bsize, int bsize_len,
+                                            const int32_t* bstride, int bstride_len,
+                                            const int32_t* boffset, int boffset_len);
+
 /*
  * Op level: replaces SparseScatterOp<GPUDevice,float,false>::Compute (sparse_gather.cc:286-357,
  * registered as "SparseScatter", sparse_gather.cc:256-268): y = copy(ybase), then the blocks of
@@ -164,13 +171,21 @@ int sbnet_sparse_gather_functor(const float* x, int N, int H, int W, int C, floa
  *   add=1, atomic=0 requires bstride >= bsize on both axes (sparse_gather.cc:322-326).
  *   add=0 with overlapping blocks: as in the reference's GPU path, which block wins on an
  *   overlapped pixel is unspecified unless the overlapping values are equal.
+ *   workspace   optional device scratch (4-byte aligned) of sbnet_sparse_scatter_workspace_bytes() bytes,
+ *               or NULL.  It only matters for add=1, atomic=1, transpose=0: with it the overlapping adds
+ *               are summed without atomics, each pixel by one owner, in ascending block-list order, so the
+ *               result is bit-identical to the reference's sequential CPU functor and several times faster
+ *               than hardware atomics.  Without it (or when more than 2x2 blocks cover a pixel, or the
+ *               list names a block twice) hardware fp32 atomics are used: same sums up to fp32
+ *               reassociation, in no particular order.
  */
 int sbnet_sparse_scatter(const float* x, int32_t num_active, const int16_t* active_block_indices,
                          const float* ybase, const int64_t* ybase_dims, int ybase_rank,
                          const int32_t* bsize, int bsize_len,
                          const int32_t* bstride, int bstride_len,
                          const int32_t* boffset, int boffset_len,
-                         int add, int atomic, int transpose, float* y, void* stream);
+                         int add, int atomic, int transpose, float* y,
+                         void* workspace, size_t workspace_bytes, void* stream);
 
 /* Op level, in place: replaces SparseScatterOp<GPUDevice,float,true>::Compute ("SparseScatterVar",
    sparse_gather.cc:242-254, 335-337).  ybase is modified and is the result. */
@@ -180,7 +195,8 @@ int sbnet_sparse_scatter_var(const float* x, int32_t num_active,
                              const int32_t* bsize, int bsize_len,
                              const int32_t* bstride, int bstride_len,
                              const int32_t* boffset, int boffset_len,
-                             int add, int atomic, int transpose, void* stream);
+                             int add, int atomic, int transpose,
+                             void* workspace, size_t workspace_bytes, void* stream);
 
 /* Functor level: replaces SparseScatterFunctor<GPUDevice,float>::operator()
    (sparse_gather.h:45-66, sparse_gather.cu:158-266).  Scatters into y in place, no validation

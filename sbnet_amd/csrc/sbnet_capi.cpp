@@ -106,7 +106,8 @@ int reduce_mask_impl(const float* mask, int N, int H, int W, const int32_t* bcou
 
 int scatter_impl(const float* x, int32_t numActive, const int16_t* idx, float* out,
                  const int64_t* dims, const int32_t* bsize, const int32_t* bstride,
-                 const int32_t* boffset, int add, int atomic, int transpose, hipStream_t stream)
+                 const int32_t* boffset, int add, int atomic, int transpose, void* workspace,
+                 size_t workspaceBytes, hipStream_t stream)
 {
     if (numActive < 0) return SBNET_EINVAL_ARG;
     if (numActive > 0 && (!x || !idx)) return SBNET_EINVAL_ARG;
@@ -116,6 +117,11 @@ int scatter_impl(const float* x, int32_t numActive, const int16_t* idx, float* o
     const sbnet::Geom g = make_geom((int)dims[0], (int)dims[1], (int)dims[2], (int)dims[3], bsize, bstride, boffset);
     const sbnet::ScatterMode mode =
         !add ? sbnet::SCATTER_ASSIGN : (atomic ? sbnet::SCATTER_ATOMIC : sbnet::SCATTER_ADD);
+    if (mode == sbnet::SCATTER_ATOMIC && !transpose && workspace) {
+        bool done = false;
+        SBNET_HIP(sbnet::launch_scatter_pull(x, out, idx, numActive, g, workspace, workspaceBytes, stream, done));
+        if (done) return SBNET_OK;
+    }
     SBNET_HIP(sbnet::launch_scatter(x, out, idx, numActive, g, transpose != 0, mode, stream));
     return SBNET_OK;
 }
@@ -213,11 +219,24 @@ int sbnet_sparse_gather_functor(const float* x, int N, int H, int W, int C, floa
     return SBNET_OK;
 }
 
+size_t sbnet_sparse_scatter_workspace_bytes(int32_t num_active, const int64_t* ybase_dims, int ybase_rank,
+                                            const int32_t* bsize, int bsize_len, const int32_t* bstride,
+                                            int bstride_len, const int32_t* boffset, int boffset_len)
+{
+    if (ybase_rank != 4 || !ybase_dims || !dims_fit_int(ybase_dims) || num_active <= 0) return 0;
+    if (!pair_ok(bsize, bsize_len) || !pair_ok(bstride, bstride_len) || !pair_ok(boffset, boffset_len)) return 0;
+    if (!geom_ok((int)ybase_dims[0], (int)ybase_dims[1], (int)ybase_dims[2], (int)ybase_dims[3], bsize, bstride))
+        return 0;
+    const sbnet::Geom g = make_geom((int)ybase_dims[0], (int)ybase_dims[1], (int)ybase_dims[2], (int)ybase_dims[3],
+                                    bsize, bstride, boffset);
+    return sbnet::scatter_pull_workspace_bytes(g, num_active);
+}
+
 int sbnet_sparse_scatter(const float* x, int32_t num_active, const int16_t* active_block_indices,
                          const float* ybase, const int64_t* ybase_dims, int ybase_rank,
                          const int32_t* bsize, int bsize_len, const int32_t* bstride, int bstride_len,
                          const int32_t* boffset, int boffset_len, int add, int atomic, int transpose,
-                         float* y, void* stream)
+                         float* y, void* workspace, size_t workspace_bytes, void* stream)
 {
     // order of checks as in sparse_gather.cc:307-327
     if (!pair_ok(bsize, bsize_len) || !pair_ok(bstride, bstride_len) || !pair_ok(boffset, boffset_len))
@@ -236,14 +255,15 @@ int sbnet_sparse_scatter(const float* x, int32_t num_active, const int16_t* acti
         return SBNET_EINVAL_ARG;
     SBNET_HIP(sbnet::launch_copy(y, ybase, count, s));  // sparse_gather.cc:338-346, no stream sync
     return scatter_impl(x, num_active, active_block_indices, y, ybase_dims, bsize, bstride, boffset, add,
-                        atomic, transpose, s);
+                        atomic, transpose, workspace, workspace_bytes, s);
 }
 
 int sbnet_sparse_scatter_var(const float* x, int32_t num_active, const int16_t* active_block_indices,
                              float* ybase, const int64_t* ybase_dims, int ybase_rank,
                              const int32_t* bsize, int bsize_len, const int32_t* bstride,
                              int bstride_len, const int32_t* boffset, int boffset_len, int add,
-                             int atomic, int transpose, void* stream)
+                             int atomic, int transpose, void* workspace, size_t workspace_bytes,
+                             void* stream)
 {
     if (!pair_ok(bsize, bsize_len) || !pair_ok(bstride, bstride_len) || !pair_ok(boffset, boffset_len))
         return SBNET_EINVAL_PARAM_SHAPE;
@@ -251,7 +271,7 @@ int sbnet_sparse_scatter_var(const float* x, int32_t num_active, const int16_t* 
     if (ybase_rank != 4) return SBNET_EINVAL_RANK;
     if (!ybase || !ybase_dims) return SBNET_EINVAL_ARG;
     return scatter_impl(x, num_active, active_block_indices, ybase, ybase_dims, bsize, bstride, boffset,
-                        add, atomic, transpose, static_cast<hipStream_t>(stream));
+                        add, atomic, transpose, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
 int sbnet_sparse_scatter_functor(const float* x, int N, int H, int W, int C, float* y, int bOffsH0,
@@ -262,7 +282,7 @@ int sbnet_sparse_scatter_functor(const float* x, int N, int H, int W, int C, flo
     const int32_t bsize[2] = {bSzH, bSzW}, bstride[2] = {bStrH, bStrW}, boffset[2] = {bOffsH0, bOffsW0};
     const int64_t dims[4] = {N, H, W, C};
     return scatter_impl(x, numActive, activeBlockIndices, y, dims, bsize, bstride, boffset, add, atomic,
-                        transpose, static_cast<hipStream_t>(stream));
+                        transpose, nullptr, 0, static_cast<hipStream_t>(stream));
 }
 
 int sbnet_copy_tensor(float* dst, const float* src, size_t count, void* stream)

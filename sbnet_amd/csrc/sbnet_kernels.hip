@@ -788,6 +788,168 @@ __global__ __launch_bounds__(256) void k_reduce_compact(const uint8_t* __restric
 }
 
 // ---------------------------------------------------------------------------------------------
+// overlapping scatter-add without atomics: every output pixel is summed by one owner
+// ---------------------------------------------------------------------------------------------
+//
+// With bstride < bsize a pixel is covered by up to ceil(R/U)*ceil(S/V) blocks.  Hardware fp32 atomics
+// resolve that at roughly a tenth of the HBM rate (every contribution is a read-modify-write in L2) and
+// in arbitrary order.  Given a little scratch memory the add is done by "pulling" instead:
+//   1. k_pull_fill / k_pull_map   an inverse map (n, bh, bw) -> position ib in the active list;
+//   2. k_pull_table               per active block, the active blocks that overlap it, sorted by ib;
+//   3. k_scatter_pull             the workgroup of block ib walks its own pixels; a pixel belongs to the
+//                                 lowest-ib block that covers it, and that owner reads the pixel once,
+//                                 adds the contributions of all covering blocks in ascending ib order
+//                                 and writes it once.
+// Ascending ib is the order in which the sequential CPU functor accumulates (sparse_gather.cc:105-129),
+// so the result is bit-identical to it and reproducible from run to run.  A block listed twice cannot
+// be represented in the map; k_pull_map notices, and k_scatter_pull then falls back to hardware atomics
+// for the whole launch (still correct, to rounding).
+
+constexpr int PULL_NB_MAX = 9;   // (2*Kh - 1) * (2*Kw - 1) with Kh = ceil(R/U), Kw = ceil(S/V) <= 2
+constexpr int PULL_LOOP = 8;     // 64-vector steps per wave
+
+struct PullArgs {
+    Geom g;
+    int bhMin, bwMin, nBH, nBW;  // extent of the inverse map: blocks that can touch the image
+    int kh1, kw1;                // Kh - 1, Kw - 1
+    int tableStride;             // ints per block in the table: 1 + 2 * NB
+    uint32_t CV, rowV, blockV;   // vectors per pixel, per block row, per block
+    uint32_t cpb, units;         // wave-units per block, in total
+    FastDiv dCpb, dRow, dCV;
+};
+
+__global__ __launch_bounds__(256) void k_pull_fill(int32_t* __restrict__ map, int64_t n, int32_t* __restrict__ dup)
+{
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) map[i] = -1;
+    if (blockIdx.x == 0 && threadIdx.x == 0) *dup = 0;
+}
+
+__device__ __forceinline__ int64_t pull_slot(const PullArgs& a, int n, int bh, int bw)
+{
+    if ((unsigned)n >= (unsigned)a.g.N) return -1;
+    const int ih = bh - a.bhMin, iw = bw - a.bwMin;
+    if ((unsigned)ih >= (unsigned)a.nBH || (unsigned)iw >= (unsigned)a.nBW) return -1;
+    return ((int64_t)n * a.nBH + ih) * a.nBW + iw;
+}
+
+__global__ __launch_bounds__(256) void k_pull_map(const int16_t* __restrict__ idx, int numActive, PullArgs a,
+                                                  int32_t* __restrict__ map, int32_t* __restrict__ dup)
+{
+    const int ib = (int)(blockIdx.x * 256 + threadIdx.x);
+    if (ib >= numActive) return;
+    const int64_t slot = pull_slot(a, idx[(size_t)ib * 3], idx[(size_t)ib * 3 + 1], idx[(size_t)ib * 3 + 2]);
+    if (slot < 0) return;  // this block cannot touch the image
+    if (atomicCAS(map + slot, -1, ib) != -1) *dup = 1;
+}
+
+__global__ __launch_bounds__(256) void k_pull_table(const int16_t* __restrict__ idx, int numActive, PullArgs a,
+                                                    const int32_t* __restrict__ map, int32_t* __restrict__ table)
+{
+    const int ib = (int)(blockIdx.x * 256 + threadIdx.x);
+    if (ib >= numActive) return;
+    const int n = idx[(size_t)ib * 3], bh = idx[(size_t)ib * 3 + 1], bw = idx[(size_t)ib * 3 + 2];
+    int ids[PULL_NB_MAX], offs[PULL_NB_MAX];
+    int cnt = 0;
+    if (pull_slot(a, n, bh, bw) >= 0) {
+        for (int dh = -a.kh1; dh <= a.kh1; ++dh)
+            for (int dw = -a.kw1; dw <= a.kw1; ++dw) {
+                const int64_t slot = pull_slot(a, n, bh + dh, bw + dw);
+                const int other = slot >= 0 ? map[slot] : -1;
+                if (other < 0) continue;
+                int k = cnt++;  // insertion sort by position in the active list
+                while (k > 0 && ids[k - 1] > other) {
+                    ids[k] = ids[k - 1];
+                    offs[k] = offs[k - 1];
+                    --k;
+                }
+                ids[k] = other;
+                offs[k] = ((dh & 0xffff) << 16) | (dw & 0xffff);
+            }
+    }
+    int32_t* t = table + (size_t)ib * a.tableStride;
+    t[0] = cnt;
+    for (int k = 0; k < cnt; ++k) {
+        t[1 + 2 * k] = ids[k];
+        t[2 + 2 * k] = offs[k];
+    }
+}
+
+// sparse_gather.cc:103-130 with add == true on overlapping blocks, NHWC stack.
+template <int VEC>
+__global__ __launch_bounds__(256) void k_scatter_pull(const float* __restrict__ x, float* __restrict__ y,
+                                                      const int16_t* __restrict__ idx, PullArgs a,
+                                                      const int32_t* __restrict__ table,
+                                                      const int32_t* __restrict__ dup)
+{
+    typedef typename Vec<VEC>::type vec;
+    const uint32_t lane = threadIdx.x & 63;
+    uint32_t unit = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (unit >= a.units) return;
+    unit = __builtin_amdgcn_readfirstlane(unit);
+    const uint32_t ib = fdiv(unit, a.dCpb);
+    const uint32_t chunk = unit - ib * a.cpb;
+    const BlockOrigin o = load_origin(idx, ib, a.g);
+    if (!o.valid) return;
+    const vec* __restrict__ xv = reinterpret_cast<const vec*>(x);
+    vec* __restrict__ yv = reinterpret_cast<vec*>(y);
+    const bool atomicMode = *dup != 0;
+    const int32_t* __restrict__ t = table + (size_t)ib * a.tableStride;
+    const int cnt = atomicMode ? 0 : t[0];
+    int ids[PULL_NB_MAX], dhs[PULL_NB_MAX], dws[PULL_NB_MAX];
+#pragma unroll
+    for (int k = 0; k < PULL_NB_MAX; ++k) {
+        ids[k] = -1;
+        dhs[k] = 0;
+        dws[k] = 0;
+        if (k < cnt) {
+            ids[k] = t[1 + 2 * k];
+            const int packed = t[2 + 2 * k];
+            dhs[k] = (int)(int16_t)(packed >> 16) * a.g.U;
+            dws[k] = (int)(int16_t)(packed & 0xffff) * a.g.V;
+        }
+    }
+
+    for (int step = 0; step < PULL_LOOP; ++step) {
+        const uint32_t e = (chunk * PULL_LOOP + step) * 64 + lane;
+        if (e >= a.blockV) break;
+        const uint32_t r = fdiv(e, a.dRow);
+        const uint32_t j = e - r * a.rowV;
+        const uint32_t s = fdiv(j, a.dCV);
+        const uint32_t cv = j - s * a.CV;
+        const int hh = o.h0 + (int)r, ww = o.w0 + (int)s;
+        if ((unsigned)hh >= (unsigned)a.g.H || (unsigned)ww >= (unsigned)a.g.W) continue;
+        vec* dst = yv + ((((int64_t)o.n * a.g.H + hh) * a.g.W + ww) * a.CV + cv);
+        if (atomicMode) {
+            commit<VEC, SCATTER_ATOMIC>(dst, ld_stream(xv + ((size_t)ib * a.blockV + e)));
+            continue;
+        }
+        // which of the overlapping blocks cover this pixel, and is this block the first of them?
+        int64_t src[PULL_NB_MAX];
+        bool first = true, mine = false;
+#pragma unroll
+        for (int k = 0; k < PULL_NB_MAX; ++k) {
+            const int rr = (int)r - dhs[k], ss = (int)s - dws[k];
+            const bool covers = ids[k] >= 0 && (unsigned)rr < (unsigned)a.g.R && (unsigned)ss < (unsigned)a.g.S;
+            src[k] = covers ? ((int64_t)ids[k] * a.blockV + (int64_t)rr * a.rowV + (int64_t)ss * a.CV + cv) : -1;
+            if (covers && first) {
+                first = false;
+                mine = ids[k] == (int)ib;
+            }
+        }
+        if (!mine) continue;
+        vec acc = ld_stream(dst);
+        vec val[PULL_NB_MAX];
+#pragma unroll
+        for (int k = 0; k < PULL_NB_MAX; ++k)
+            if (src[k] >= 0) val[k] = ld_stream(xv + src[k]);
+#pragma unroll
+        for (int k = 0; k < PULL_NB_MAX; ++k)
+            if (src[k] >= 0) acc = vadd(acc, val[k]);
+        st_stream(dst, acc);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // flat copy (CopyTensorFunctor, sparse_gather.cc:135-142 / sparse_gather.cu:268-276)
 // ---------------------------------------------------------------------------------------------
 
@@ -1090,6 +1252,80 @@ hipError_t launch_scatter(const float* x, float* y, const int16_t* idx, int numA
     else if (vec == 2) scatter_mode<2>(x, y, idx, g, numActive, transpose, mode, stream, err);
     else scatter_mode<1>(x, y, idx, g, numActive, transpose, mode, stream, err);
     if (err != hipSuccess) return err;
+    return hipGetLastError();
+}
+
+// Geometry of the inverse block map of the pull scatter; false when the method does not apply.
+static bool make_pull_args(const Geom& g, int numActive, int vec, PullArgs& a, int64_t& mapN)
+{
+    a.g = g;
+    const int Kh = (g.R + g.U - 1) / g.U, Kw = (g.S + g.V - 1) / g.V;
+    if ((2 * Kh - 1) * (2 * Kw - 1) > PULL_NB_MAX) return false;
+    a.kh1 = Kh - 1;
+    a.kw1 = Kw - 1;
+    a.tableStride = 1 + 2 * (2 * Kh - 1) * (2 * Kw - 1);
+    // blocks that can touch the image: oh + bh*U + R - 1 >= 0 and oh + bh*U <= H - 1 (floor divisions)
+    auto floordiv = [](int64_t p, int64_t q) { return p >= 0 ? p / q : -((-p + q - 1) / q); };
+    int64_t bhMin = -floordiv((int64_t)g.R - 1 + g.oh, g.U), bhMax = floordiv((int64_t)g.H - 1 - g.oh, g.U);
+    int64_t bwMin = -floordiv((int64_t)g.S - 1 + g.ow, g.V), bwMax = floordiv((int64_t)g.W - 1 - g.ow, g.V);
+    if (bhMin < -32768) bhMin = -32768;
+    if (bwMin < -32768) bwMin = -32768;
+    if (bhMax > 32767) bhMax = 32767;
+    if (bwMax > 32767) bwMax = 32767;
+    if (bhMax < bhMin || bwMax < bwMin) return false;
+    a.bhMin = (int)bhMin; a.bwMin = (int)bwMin;
+    a.nBH = (int)(bhMax - bhMin + 1); a.nBW = (int)(bwMax - bwMin + 1);
+    mapN = (int64_t)g.N * a.nBH * a.nBW;
+    if (mapN >= (1ll << 31)) return false;
+    const uint64_t rowV = (uint64_t)g.S * g.C / vec, blockV = rowV * g.R;
+    if (blockV >= (1ull << 31)) return false;
+    a.CV = (uint32_t)(g.C / vec);
+    a.rowV = (uint32_t)rowV;
+    a.blockV = (uint32_t)blockV;
+    a.cpb = (uint32_t)((blockV + 64 * PULL_LOOP - 1) / (64 * PULL_LOOP));
+    const uint64_t units = (uint64_t)numActive * a.cpb;
+    if (units >= (1ull << 31)) return false;
+    a.units = (uint32_t)units;
+    a.dCpb = make_fastdiv(a.cpb);
+    a.dRow = make_fastdiv(a.rowV);
+    a.dCV = make_fastdiv(a.CV);
+    return true;
+}
+
+size_t scatter_pull_workspace_bytes(const Geom& g, int numActive)
+{
+    PullArgs a;
+    int64_t mapN = 0;
+    if (numActive <= 0 || !make_pull_args(g, numActive, 1, a, mapN)) return 0;
+    return (size_t)mapN * 4 + 16 + (size_t)numActive * a.tableStride * 4;
+}
+
+hipError_t launch_scatter_pull(const float* x, float* y, const int16_t* idx, int numActive, const Geom& g,
+                               void* workspace, size_t workspaceBytes, hipStream_t stream, bool& done)
+{
+    done = false;
+    if (numActive == 0) { done = true; return hipSuccess; }
+    PullArgs a;
+    int64_t mapN = 0;
+    const int vec = pick_vec(g, y, x);
+    if (!workspace || !make_pull_args(g, numActive, vec, a, mapN)) return hipSuccess;
+    if (workspaceBytes < scatter_pull_workspace_bytes(g, numActive) || (reinterpret_cast<uintptr_t>(workspace) & 3))
+        return hipSuccess;
+    int32_t* map = static_cast<int32_t*>(workspace);
+    int32_t* dup = map + mapN;
+    int32_t* table = dup + 4;
+    int64_t fillWgs = (mapN + 255) / 256;
+    if (fillWgs > 4096) fillWgs = 4096;
+    if (fillWgs < 1) fillWgs = 1;
+    const unsigned perBlockWgs = (unsigned)((numActive + 255) / 256);
+    hipLaunchKernelGGL(k_pull_fill, dim3((unsigned)fillWgs), dim3(256), 0, stream, map, mapN, dup);
+    hipLaunchKernelGGL(k_pull_map, dim3(perBlockWgs), dim3(256), 0, stream, idx, numActive, a, map, dup);
+    hipLaunchKernelGGL(k_pull_table, dim3(perBlockWgs), dim3(256), 0, stream, idx, numActive, a, map, table);
+    const unsigned wgs = (a.units + 3) / 4;
+    if (vec == 4) hipLaunchKernelGGL(k_scatter_pull<4>, dim3(wgs), dim3(256), 0, stream, x, y, idx, a, table, dup);
+    else if (vec == 2) hipLaunchKernelGGL(k_scatter_pull<2>, dim3(wgs), dim3(256), 0, stream, x, y, idx, a, table, dup);
+    else hipLaunchKernelGGL(k_scatter_pull<1>, dim3(wgs), dim3(256), 0, stream, x, y, idx, a, table, dup);
+    done = true;
     return hipGetLastError();
 }
 

@@ -33,6 +33,13 @@ hipError_t launch_gather(const float* x, float* y, const int16_t* idx, int numAc
 hipError_t launch_scatter(const float* x, float* y, const int16_t* idx, int numActive,
                           const Geom& g, bool transpose, ScatterMode mode, hipStream_t stream);
 
+// Scatter-add on overlapping blocks without atomics (NHWC stack only): bit-identical to the sequential CPU
+// order.  Needs scratch of scatter_pull_workspace_bytes(); `done` is false when the method does not apply
+// (no or too little scratch, more than 2x2 blocks covering a pixel) and nothing was launched.
+size_t scatter_pull_workspace_bytes(const Geom& g, int numActive);
+hipError_t launch_scatter_pull(const float* x, float* y, const int16_t* idx, int numActive, const Geom& g,
+                               void* workspace, size_t workspaceBytes, hipStream_t stream, bool& done);
+
 hipError_t launch_copy(float* dst, const float* src, size_t count, hipStream_t stream);
 
 }  // namespace sbnet

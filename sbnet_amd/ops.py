@@ -159,15 +159,22 @@ def _scatter(x, bin_counts, active_block_indices, ybase, dynamic_bsize, dynamic_
     bo, bop, bol = _pair(dynamic_boffset)
     dims, rank = _dims(ybase)
     with torch.cuda.device(ybase.device):
+        ws_ptr, ws_bytes = None, 0
+        if add and atomic and not transpose:
+            # scratch for the atomic-free, order-preserving scatter-add of overlapping blocks
+            need = lib.sbnet_sparse_scatter_workspace_bytes(M, dims, rank, bsp, bsl, btp, btl, bop, bol)
+            if need:
+                ws = _workspace(ybase.device, need)
+                ws_ptr, ws_bytes = ws.data_ptr(), ws.numel()
         if use_var:
             _check(lib.sbnet_sparse_scatter_var(x.data_ptr(), M, idx.data_ptr(), ybase.data_ptr(), dims, rank,
                                                 bsp, bsl, btp, btl, bop, bol, int(bool(add)), int(bool(atomic)),
-                                                int(bool(transpose)), _stream()))
+                                                int(bool(transpose)), ws_ptr, ws_bytes, _stream()))
             return ybase
         y = torch.empty_like(ybase)
         _check(lib.sbnet_sparse_scatter(x.data_ptr(), M, idx.data_ptr(), ybase.data_ptr(), dims, rank, bsp, bsl,
                                         btp, btl, bop, bol, int(bool(add)), int(bool(atomic)),
-                                        int(bool(transpose)), y.data_ptr(), _stream()))
+                                        int(bool(transpose)), y.data_ptr(), ws_ptr, ws_bytes, _stream()))
         return y
 
 

@@ -50,6 +50,19 @@ def test_size_queries():
     assert lib.sbnet_reduce_mask_workspace_bytes(4, I32x3(1, 1, 1), 3) == 0
 
 
+def test_scatter_workspace_query():
+    lib = _lib.load()
+    dims = I64x4(2, 512, 512, 256)
+    # 16x16 blocks at stride 8: 2x2 blocks cover a pixel, the atomic-free method applies
+    n = lib.sbnet_sparse_scatter_workspace_bytes(2000, dims, 4, I32x2(16, 16), 2, I32x2(8, 8), 2, I32x2(0, 0), 2)
+    assert n >= 2 * 64 * 64 * 4 + 2000 * 4
+    # 16x16 at stride 4: 4x4 blocks cover a pixel, it does not
+    assert lib.sbnet_sparse_scatter_workspace_bytes(2000, dims, 4, I32x2(16, 16), 2, I32x2(4, 4), 2, I32x2(0, 0),
+                                                    2) == 0
+    assert lib.sbnet_sparse_scatter_workspace_bytes(2000, dims, 3, I32x2(16, 16), 2, I32x2(8, 8), 2, I32x2(0, 0),
+                                                    2) == 0
+
+
 def test_reduce_mask_param_shape_errors():
     lib = _lib.load()
     ok = I32x2(2, 2)
@@ -104,9 +117,9 @@ def test_scatter_errors(var):
     def call(rank, bstride, blen, add, atomic):
         if var:
             return lib.sbnet_sparse_scatter_var(FAKE, 1, FAKE, FAKE, dims, rank, size, 2, bstride, blen, ok, 2, add,
-                                                atomic, 0, None)
+                                                atomic, 0, None, 0, None)
         return lib.sbnet_sparse_scatter(FAKE, 1, FAKE, FAKE, dims, rank, size, 2, bstride, blen, ok, 2, add, atomic,
-                                        0, ctypes.c_void_p(0x100000), None)
+                                        0, ctypes.c_void_p(0x100000), None, 0, None)
 
     assert call(4, overlap, 2, 1, 0) == _lib.SBNET_EINVAL_OVERLAP      # sparse_gather.cc:322-326
     assert call(3, overlap, 2, 1, 0) == _lib.SBNET_EINVAL_OVERLAP      # tested before the rank
@@ -120,7 +133,7 @@ def test_scatter_rejects_aliasing_output():
     dims = I64x4(1, 4, 4, 1)
     ok = I32x2(2, 2)
     rc = lib.sbnet_sparse_scatter(FAKE, 1, FAKE, FAKE, dims, 4, ok, 2, ok, 2, ok, 2, 0, 0, 0,
-                                  ctypes.c_void_p(0x1000 + 16), None)
+                                  ctypes.c_void_p(0x1000 + 16), None, 0, None)
     assert rc == _lib.SBNET_EINVAL_ARG
 
 
