@@ -48,6 +48,9 @@ def parse():
     ap.add_argument("--density", type=float, default=0.30)
     ap.add_argument("--all-configs", action="store_true")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline (profiling runs)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run the library's plain copy kernel on 256 MiB, 10 times: a kernel of known traffic "
+                         "against which profiler byte counters are scaled")
     return ap.parse_args()
 
 
@@ -289,6 +292,18 @@ def main():
     from sbnet_amd import _lib, workloads
     lib = _lib.load()
     torch.cuda.set_device(0)
+
+    if args.copy_calibration:
+        n = 64 * 1024 * 1024  # floats: 256 MiB read + 256 MiB written per launch
+        src = [torch.ones(n, device="cuda:0") for _ in range(3)]
+        dst = [torch.empty(n, device="cuda:0") for _ in range(3)]
+        st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        for i in range(10):
+            rc = lib.sbnet_copy_tensor(dst[i % 3].data_ptr(), src[i % 3].data_ptr(), n, st)
+            assert rc == 0
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
 
     wl = workloads.config3(args.density)
     path = Path(wl, torch, lib, nsets=3)
