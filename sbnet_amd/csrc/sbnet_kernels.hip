@@ -121,27 +121,33 @@ __device__ __forceinline__ BlockOrigin load_origin(const int16_t* __restrict__ i
 // The same in two steps, for software pipelines: the loads are issued early and the arithmetic (which
 // is what makes a wave wait for them) happens where the origin is first needed.
 struct RawTriple {
-    uint32_t nbh;  // n in the low half, bh in the high half, exactly as loaded
-    int bw;
+    uint32_t lo, hi;  // the two aligned dwords that hold the 6-byte triple
+    uint32_t shift;   // 0 or 16: where the triple starts inside them
 };
 
-typedef uint32_t u32_a2 __attribute__((aligned(2)));
-
+// ib is the same for the whole workgroup.  Reading the two aligned dwords around the triple from a uniform
+// address lets the compiler use the scalar unit, whose loads are counted apart from vector loads and stores:
+// waiting for the triple then does not wait for the stores in flight.  (A triple that ends the list on a
+// 4-byte boundary + 2 makes the second dword reach 2 bytes past the list, inside the same aligned dword.)
 __device__ __forceinline__ RawTriple load_triple(const int16_t* __restrict__ idx, uint32_t ib)
 {
-    const int16_t* t = idx + (size_t)ib * 3;
+    const uint32_t byteOff = 6u * (uint32_t)__builtin_amdgcn_readfirstlane(ib);
+    const uintptr_t base = reinterpret_cast<uintptr_t>(idx) + byteOff;
+    const uint32_t* __restrict__ w = reinterpret_cast<const uint32_t*>(base & ~(uintptr_t)3);
     RawTriple r;
-    r.nbh = *reinterpret_cast<const u32_a2*>(t);
-    r.bw = t[2];
+    r.lo = w[0];
+    r.hi = w[1];
+    r.shift = (uint32_t)(base & 2) * 8u;
     return r;
 }
 
 __device__ __forceinline__ BlockOrigin origin_of(const RawTriple& r, const Geom& g)
 {
+    const uint64_t bits = (((uint64_t)r.hi << 32) | r.lo) >> r.shift;
     BlockOrigin o;
-    o.n = (int)(int16_t)(r.nbh & 0xffffu);
-    o.h0 = g.oh + (int)(int16_t)(r.nbh >> 16) * g.U;
-    o.w0 = g.ow + r.bw * g.V;
+    o.n = (int)(int16_t)(bits & 0xffffu);
+    o.h0 = g.oh + (int)(int16_t)((bits >> 16) & 0xffffu) * g.U;
+    o.w0 = g.ow + (int)(int16_t)((bits >> 32) & 0xffffu) * g.V;
     o.valid = (unsigned)o.n < (unsigned)g.N;
     return o;
 }
@@ -311,6 +317,7 @@ struct TileArgs {
     uint32_t total;     // numActive * tpb
     uint32_t tilesPerWg;
     uint32_t vpr;       // slots per planar row: (P + 3) / 4
+    uint32_t dbg;       // experiments only: bit0 skip NHWC loads, bit1 skip planar stores
     FastDiv dTpb, dPs, dS, dVpr;
 };
 
@@ -332,6 +339,15 @@ __device__ __forceinline__ void decode_tile(const TileArgs& a, uint32_t id, Tile
 }
 
 __device__ __forceinline__ uint32_t lds_swz(uint32_t c) { return ((c >> 2) & 7u) << 2; }
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits until every global store of
+// the wave has been acknowledged (vmcnt(0)), which would drain the store queue once per tile.
+__device__ __forceinline__ void lds_barrier()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
 
 // NHWC side, global -> registers.  Vector i = u*nthr + tid of the tile is pixel i >> lppLog, channel
 // vector i & (lpp - 1).  Pixels outside the image read as zero (sparse_gather.cc:80-82).
@@ -356,30 +372,42 @@ __device__ __forceinline__ void nhwc_load_tile(const typename Vec<VEC>::type* __
         const int hh = o.h0 + (int)r, ww = o.w0 + (int)(p - r * a.g.S);
         const int c = t.c0 + (int)cl * VEC;
         const bool ok = i < items && o.valid && (unsigned)hh < (unsigned)a.g.H && (unsigned)ww < (unsigned)a.g.W &&
-                        c < a.g.C;
+                        c < a.g.C && !(a.dbg & 1);
         const int64_t src = (((int64_t)o.n * a.g.H + hh) * a.g.W + ww) * CV + (c / VEC);
         v[u] = *reinterpret_cast<const vec*>(reinterpret_cast<const char*>(xv) + (ok ? src * (int64_t)sizeof(vec) : zoff));
     }
 }
 
-// Planar side, LDS -> global: slot i of the tile is row i / vpr, floats [4v, 4v + 4) of its run.
+// Planar side, LDS -> global: slot i of the tile is row i / vpr, floats [4v, 4v + 4) of its run.  LDS reads
+// are batched four deep ahead of the stores so that their latency is paid once per batch, not per slot.
 __device__ __forceinline__ void planar_store_tile(float* __restrict__ g0, int64_t RS, const float* __restrict__ lds,
                                                   const TileArgs& a, const TileId& t, uint32_t tid, uint32_t nthr)
 {
     const uint32_t items = (uint32_t)t.ctEff * a.vpr;
-    for (uint32_t i = tid; i < items; i += nthr) {
-        const uint32_t c = fdiv(i, a.dVpr);
-        const uint32_t v = i - c * a.vpr;
-        const int e0 = 4 * (int)v;
-        if (e0 >= t.Pn) continue;
-        const f4 q = *reinterpret_cast<const f4*>(lds + c * a.Pp + ((4u * v) ^ lds_swz(c)));
-        float* __restrict__ dst = g0 + (int64_t)c * RS + e0;
-        if (e0 + 4 <= t.Pn) {
-            __builtin_nontemporal_store(q, reinterpret_cast<f4u*>(dst));
-        } else {
-            dst[0] = q.x;
-            if (e0 + 1 < t.Pn) dst[1] = q.y;
-            if (e0 + 2 < t.Pn) dst[2] = q.z;
+    for (uint32_t base = 0; base < items; base += 4 * nthr) {
+        f4 q[4];
+        float* dst[4];
+        int left[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const uint32_t i = base + u * nthr + tid;
+            const uint32_t c = fdiv(i, a.dVpr);
+            const uint32_t v = i - c * a.vpr;
+            const int e0 = 4 * (int)v;
+            left[u] = i < items ? t.Pn - e0 : 0;  // floats of the run from this slot on; <= 0: nothing to store
+            const bool live = left[u] > 0;
+            q[u] = *reinterpret_cast<const f4*>(lds + (live ? c * a.Pp + ((4u * v) ^ lds_swz(c)) : 0u));
+            dst[u] = g0 + (int64_t)c * RS + e0;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (left[u] >= 4) {
+                __builtin_nontemporal_store(q[u], reinterpret_cast<f4u*>(dst[u]));
+            } else if (left[u] > 0) {
+                dst[u][0] = q[u].x;
+                if (left[u] > 1) dst[u][1] = q[u].y;
+                if (left[u] > 2) dst[u][2] = q[u].z;
+            }
         }
     }
 }
@@ -416,23 +444,27 @@ __global__ __launch_bounds__(256) void k_gather_planar(const float* __restrict__
     const int64_t RS = (int64_t)a.g.R * a.g.S;
     const vec* __restrict__ xv = reinterpret_cast<const vec*>(x);
 
-    // Pipeline state: `cur` is in registers (v) on its way to LDS, `nxt` is the tile whose loads are
-    // issued while `cur` is stored; block triples are fetched one tile further ahead so that no wave
-    // ever waits on an index load with nothing else in flight.
-    TileId cur, nxt;
+    // Pipeline state: `cur` is in registers (v) on its way to LDS; the loads of the following tile are
+    // issued while `cur` is being stored.
+    TileId cur;
     decode_tile(a, tile, cur);
     vec v[TILE_LD];
     nhwc_load_tile<VEC>(xv, a, cur, load_origin(idx, cur.ib, a.g), tid, nthr, v);
-    bool more = tile + 1 < tileEnd;
-    nxt = cur;
-    RawTriple rawNext = {0u, 0};
-    if (more) {
-        decode_tile(a, tile + 1, nxt);
-        rawNext = load_triple(idx, nxt.ib);
-    }
 
     for (;;) {
+        const bool more = tile + 1 < tileEnd;
+        TileId nxt = cur;
+        RawTriple rawNext = {0u, 0u, 0u};
+        if (more) {
+            // scalar load, issued a whole LDS phase and store phase before its result is needed
+            decode_tile(a, tile + 1, nxt);
+            rawNext = load_triple(idx, nxt.ib);
+        }
         const uint32_t items = (uint32_t)cur.Pn << a.lppLog;
+        // vmcnt(0): every lane waits for its tile loads here, also lanes that skip all the LDS writes below;
+        // otherwise the compiler has to assume loads still pending further down and waits there, behind the
+        // stores (s_waitcnt immediate: vmcnt 0, expcnt and lgkmcnt untouched)
+        __builtin_amdgcn_s_waitcnt(0x0F70);
 #pragma unroll
         for (int u = 0; u < TILE_LD; ++u) {
             const uint32_t i = u * nthr + tid;
@@ -445,27 +477,16 @@ __global__ __launch_bounds__(256) void k_gather_planar(const float* __restrict__
                 }
             }
         }
-        __syncthreads();
+        lds_barrier();
         float* __restrict__ g0 = y + ((int64_t)cur.ib * a.g.C + cur.c0) * RS + cur.p0;
-        TileId nn = nxt;
-        RawTriple rawNn = rawNext;
-        const bool more2 = tile + 2 < tileEnd;
-        if (more) nhwc_load_tile<VEC>(xv, a, nxt, origin_of(rawNext, a.g), tid, nthr, v);
-        planar_store_tile(g0, RS, lds, a, cur, tid, nthr);
+        // Stores of this tile first, loads of the next tile after them: vector memory operations retire in
+        // order, so the wait for the loads at the top of the loop then covers nothing younger than them.
+        if (!(a.dbg & 2)) planar_store_tile(g0, RS, lds, a, cur, tid, nthr);
         if (!more) break;
-        // The triple of the tile after next is fetched last: the wave makes it uniform at once, which
-        // waits for it, and memory operations retire in order - issued before the tile loads it would
-        // make every wave wait for those loads here instead of at the top of the loop.
-        if (more2) {
-            decode_tile(a, tile + 2, nn);
-            rawNn = load_triple(idx, nn.ib);
-        }
-        __syncthreads();
+        nhwc_load_tile<VEC>(xv, a, nxt, origin_of(rawNext, a.g), tid, nthr, v);
+        lds_barrier();
         ++tile;
         cur = nxt;
-        nxt = nn;
-        rawNext = rawNn;
-        more = more2;
     }
 }
 
@@ -487,12 +508,13 @@ __global__ __launch_bounds__(256) void k_scatter_planar(const float* __restrict_
 
     TileId cur;
     decode_tile(a, tile, cur);
-    RawTriple raw = load_triple(idx, cur.ib);  // consumed after the planar loads below have landed
     f4 val[TILE_LD];
     planar_load_tile(x + ((int64_t)cur.ib * a.g.C + cur.c0) * RS + cur.p0, RS, a, cur, tid, nthr, val);
 
     for (;;) {
+        const RawTriple raw = load_triple(idx, cur.ib);  // scalar load, needed only after the barrier below
         const uint32_t slots = (uint32_t)cur.ctEff * a.vpr;
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), see k_gather_planar
 #pragma unroll
         for (int u = 0; u < TILE_LD; ++u) {
             const uint32_t i = u * nthr + tid;
@@ -512,16 +534,13 @@ __global__ __launch_bounds__(256) void k_scatter_planar(const float* __restrict_
                 }
             }
         }
-        __syncthreads();
+        lds_barrier();
         const bool more = tile + 1 < tileEnd;
         const TileId done = cur;
         const BlockOrigin od = origin_of(raw, a.g);
-        if (more) {
-            decode_tile(a, tile + 1, cur);
-            planar_load_tile(x + ((int64_t)cur.ib * a.g.C + cur.c0) * RS + cur.p0, RS, a, cur, tid, nthr, val);
-        }
         // NHWC side of the finished tile: LDS -> base tensor; pixels outside the image are dropped
-        // (sparse_gather.cc:121).
+        // (sparse_gather.cc:121).  The loads of the next tile are issued after these stores (k_gather_planar
+        // says why).
         if (od.valid) {
             const uint32_t items = (uint32_t)done.Pn << a.lppLog;
             for (uint32_t base = 0; base < items; base += nthr * 4) {
@@ -564,8 +583,9 @@ __global__ __launch_bounds__(256) void k_scatter_planar(const float* __restrict_
             }
         }
         if (!more) break;
-        raw = load_triple(idx, cur.ib);  // after the stores, see k_gather_planar
-        __syncthreads();
+        decode_tile(a, tile + 1, cur);
+        planar_load_tile(x + ((int64_t)cur.ib * a.g.C + cur.c0) * RS + cur.p0, RS, a, cur, tid, nthr, val);
+        lds_barrier();
         ++tile;
     }
 }
@@ -997,7 +1017,7 @@ static uint32_t pow2_ceil(uint32_t v)
 
 // Optional overrides for experiments: SBNET_TUNE="ct=32,lds=32768,occ=4".
 struct Tune {
-    int ct = 0, ldsBytes = 0, wg = 0, occ = 0;
+    int ct = 0, ldsBytes = 0, wg = 0, occ = 0, dbg = 0;
 };
 
 static Tune read_tune()
@@ -1010,6 +1030,7 @@ static Tune read_tune()
     if ((p = strstr(s, "lds="))) t.ldsBytes = atoi(p + 4);
     if ((p = strstr(s, "wg="))) t.wg = atoi(p + 3);
     if ((p = strstr(s, "occ="))) t.occ = atoi(p + 4);
+    if ((p = strstr(s, "dbg="))) t.dbg = atoi(p + 4);
     return t;
 }
 
@@ -1146,6 +1167,7 @@ static bool make_tile_args(const Geom& g, int numActive, int vec, TileArgs& a, i
     a.psplit = (RS + a.P - 1) / a.P;
     a.Pp = (a.P + 31) / 32 * 32;
     a.vpr = (uint32_t)((a.P + 3) / 4);
+    a.dbg = (uint32_t)tune.dbg;
     a.tpb = (uint32_t)(a.psplit * a.cchunks);
     const uint64_t total = (uint64_t)numActive * a.tpb;
     if (total >= (1ull << 31)) return false;
