@@ -285,15 +285,15 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
 // at the speed of aligned ones (measured with a plain copy), which makes an aligned-body / scalar-
 // head-and-tail split unnecessary.  Only the last slot of a run can be partial.
 //
-// Workgroups are persistent: each takes a contiguous range of tiles and software-pipelines them.
-// The global loads of tile i+1 are issued into registers before the stores of tile i leave LDS, so
-// a workgroup keeps reads and writes in flight at the same time instead of alternating between a
-// load phase and a store phase.  To keep that pipeline free of control flow around loads (which
-// would force the compiler to wait for each load where the branches join), every load is issued
-// unconditionally from an address that is always valid, and a bit mask remembers which registers
-// hold real data.  Tiles are ordered (block, channel chunk, pixel split) with the pixel split
-// fastest: the splits of one channel chunk continue each other's planar runs, and a workgroup that
-// owns them back to back lets the 128-byte lines shared at the seams merge in its XCD's L2.
+// One workgroup moves one tile: all of its global loads are issued back to back into registers (no
+// control flow around them: out-of-image pixels read a 16-byte zero buffer, lanes past the end of the
+// tile a valid dummy address), then go through LDS, then leave as stores.  A persistent variant that
+// software-pipelined several tiles per workgroup (loads of tile i+1 in flight during the stores of tile
+// i) was measured slower the more tiles a workgroup owned (47 -> 52 -> 65 us for 1, 4, 12 tiles per
+// workgroup on the 800x800x128 workload): the hardware dispatcher balances one-tile workgroups better
+// than a static split, and with 4-5 workgroups resident per CU their phases overlap anyway.  Tiles are
+// numbered (block, channel chunk, pixel split) with the pixel split fastest, so the splits of one
+// channel chunk, which continue each other's planar runs, are dispatched together.
 //
 // LDS layout: tile row c at c*Pp floats, Pp a multiple of 32, pixel e at column e.  Columns are
 // XOR-swizzled in units of 4 floats by ((c >> 2) & 7): the planar side still sees aligned groups of
@@ -315,9 +315,7 @@ struct TileArgs {
     int cchunks;        // channel chunks per block
     uint32_t tpb;       // tiles per block = psplit * cchunks
     uint32_t total;     // numActive * tpb
-    uint32_t tilesPerWg;
     uint32_t vpr;       // slots per planar row: (P + 3) / 4
-    uint32_t dbg;       // experiments only: bit0 skip NHWC loads, bit1 skip planar stores
     FastDiv dTpb, dPs, dS, dVpr;
 };
 
@@ -372,7 +370,7 @@ __device__ __forceinline__ void nhwc_load_tile(const typename Vec<VEC>::type* __
         const int hh = o.h0 + (int)r, ww = o.w0 + (int)(p - r * a.g.S);
         const int c = t.c0 + (int)cl * VEC;
         const bool ok = i < items && o.valid && (unsigned)hh < (unsigned)a.g.H && (unsigned)ww < (unsigned)a.g.W &&
-                        c < a.g.C && !(a.dbg & 1);
+                        c < a.g.C;
         const int64_t src = (((int64_t)o.n * a.g.H + hh) * a.g.W + ww) * CV + (c / VEC);
         v[u] = *reinterpret_cast<const vec*>(reinterpret_cast<const char*>(xv) + (ok ? src * (int64_t)sizeof(vec) : zoff));
     }
@@ -437,57 +435,29 @@ __global__ __launch_bounds__(256) void k_gather_planar(const float* __restrict__
     typedef typename Vec<VEC>::type vec;
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const uint32_t tid = threadIdx.x, nthr = blockDim.x;
-    uint32_t tile = blockIdx.x * a.tilesPerWg;
-    const uint32_t tileEnd = min(a.total, tile + a.tilesPerWg);
-    if (tile >= tileEnd) return;
     const uint32_t lppMask = (1u << a.lppLog) - 1u;
     const int64_t RS = (int64_t)a.g.R * a.g.S;
-    const vec* __restrict__ xv = reinterpret_cast<const vec*>(x);
+    TileId t;
+    decode_tile(a, blockIdx.x, t);
 
-    // Pipeline state: `cur` is in registers (v) on its way to LDS; the loads of the following tile are
-    // issued while `cur` is being stored.
-    TileId cur;
-    decode_tile(a, tile, cur);
     vec v[TILE_LD];
-    nhwc_load_tile<VEC>(xv, a, cur, load_origin(idx, cur.ib, a.g), tid, nthr, v);
+    nhwc_load_tile<VEC>(reinterpret_cast<const vec*>(x), a, t, origin_of(load_triple(idx, t.ib), a.g), tid, nthr, v);
 
-    for (;;) {
-        const bool more = tile + 1 < tileEnd;
-        TileId nxt = cur;
-        RawTriple rawNext = {0u, 0u, 0u};
-        if (more) {
-            // scalar load, issued a whole LDS phase and store phase before its result is needed
-            decode_tile(a, tile + 1, nxt);
-            rawNext = load_triple(idx, nxt.ib);
-        }
-        const uint32_t items = (uint32_t)cur.Pn << a.lppLog;
-        // vmcnt(0): every lane waits for its tile loads here, also lanes that skip all the LDS writes below;
-        // otherwise the compiler has to assume loads still pending further down and waits there, behind the
-        // stores (s_waitcnt immediate: vmcnt 0, expcnt and lgkmcnt untouched)
-        __builtin_amdgcn_s_waitcnt(0x0F70);
+    const uint32_t items = (uint32_t)t.Pn << a.lppLog;
 #pragma unroll
-        for (int u = 0; u < TILE_LD; ++u) {
-            const uint32_t i = u * nthr + tid;
-            if (i < items) {
-                const uint32_t pl = i >> a.lppLog, cl = i & lppMask;
+    for (int u = 0; u < TILE_LD; ++u) {
+        const uint32_t i = u * nthr + tid;
+        if (i < items) {
+            const uint32_t pl = i >> a.lppLog, cl = i & lppMask;
 #pragma unroll
-                for (int k = 0; k < VEC; ++k) {
-                    const uint32_t c = cl * VEC + k;
-                    lds[c * a.Pp + (pl ^ lds_swz(c))] = vget(v[u], k);
-                }
+            for (int k = 0; k < VEC; ++k) {
+                const uint32_t c = cl * VEC + k;
+                lds[c * a.Pp + (pl ^ lds_swz(c))] = vget(v[u], k);
             }
         }
-        lds_barrier();
-        float* __restrict__ g0 = y + ((int64_t)cur.ib * a.g.C + cur.c0) * RS + cur.p0;
-        // Stores of this tile first, loads of the next tile after them: vector memory operations retire in
-        // order, so the wait for the loads at the top of the loop then covers nothing younger than them.
-        if (!(a.dbg & 2)) planar_store_tile(g0, RS, lds, a, cur, tid, nthr);
-        if (!more) break;
-        nhwc_load_tile<VEC>(xv, a, nxt, origin_of(rawNext, a.g), tid, nthr, v);
-        lds_barrier();
-        ++tile;
-        cur = nxt;
     }
+    lds_barrier();
+    planar_store_tile(y + ((int64_t)t.ib * a.g.C + t.c0) * RS + t.p0, RS, lds, a, t, tid, nthr);
 }
 
 // sparse_gather.cc:103-130 with transpose == true: the block stack is [blocks, C, R, S].
@@ -498,95 +468,80 @@ __global__ __launch_bounds__(256) void k_scatter_planar(const float* __restrict_
     typedef typename Vec<VEC>::type vec;
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const uint32_t tid = threadIdx.x, nthr = blockDim.x;
-    uint32_t tile = blockIdx.x * a.tilesPerWg;
-    const uint32_t tileEnd = min(a.total, tile + a.tilesPerWg);
-    if (tile >= tileEnd) return;
     const uint32_t lppMask = (1u << a.lppLog) - 1u;
     const int64_t RS = (int64_t)a.g.R * a.g.S;
     vec* __restrict__ yv = reinterpret_cast<vec*>(y);
     const int CV = a.g.C / VEC;
+    TileId t;
+    decode_tile(a, blockIdx.x, t);
+    const RawTriple raw = load_triple(idx, t.ib);  // scalar load, needed only after the barrier
 
-    TileId cur;
-    decode_tile(a, tile, cur);
     f4 val[TILE_LD];
-    planar_load_tile(x + ((int64_t)cur.ib * a.g.C + cur.c0) * RS + cur.p0, RS, a, cur, tid, nthr, val);
+    planar_load_tile(x + ((int64_t)t.ib * a.g.C + t.c0) * RS + t.p0, RS, a, t, tid, nthr, val);
 
-    for (;;) {
-        const RawTriple raw = load_triple(idx, cur.ib);  // scalar load, needed only after the barrier below
-        const uint32_t slots = (uint32_t)cur.ctEff * a.vpr;
-        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), see k_gather_planar
+    const uint32_t slots = (uint32_t)t.ctEff * a.vpr;
 #pragma unroll
-        for (int u = 0; u < TILE_LD; ++u) {
-            const uint32_t i = u * nthr + tid;
-            if (i < slots) {
-                const uint32_t c = fdiv(i, a.dVpr);
-                const uint32_t vs = i - c * a.vpr;
-                const int e0 = 4 * (int)vs;
-                float* __restrict__ row = lds + c * a.Pp;
-                if (e0 + 4 <= cur.Pn) {
-                    *reinterpret_cast<f4*>(row + ((uint32_t)e0 ^ lds_swz(c))) = val[u];
-                } else if (e0 < cur.Pn) {  // partial last slot: holds floats [Pn-4, Pn) of the run
-                    const uint32_t t0 = (uint32_t)(cur.Pn - 4);
-                    row[(t0 + 0) ^ lds_swz(c)] = val[u].x;
-                    row[(t0 + 1) ^ lds_swz(c)] = val[u].y;
-                    row[(t0 + 2) ^ lds_swz(c)] = val[u].z;
-                    row[(t0 + 3) ^ lds_swz(c)] = val[u].w;
-                }
+    for (int u = 0; u < TILE_LD; ++u) {
+        const uint32_t i = u * nthr + tid;
+        if (i < slots) {
+            const uint32_t c = fdiv(i, a.dVpr);
+            const uint32_t vs = i - c * a.vpr;
+            const int e0 = 4 * (int)vs;
+            float* __restrict__ row = lds + c * a.Pp;
+            if (e0 + 4 <= t.Pn) {
+                *reinterpret_cast<f4*>(row + ((uint32_t)e0 ^ lds_swz(c))) = val[u];
+            } else if (e0 < t.Pn) {  // partial last slot: holds floats [Pn-4, Pn) of the run
+                const uint32_t t0 = (uint32_t)(t.Pn - 4);
+                row[(t0 + 0) ^ lds_swz(c)] = val[u].x;
+                row[(t0 + 1) ^ lds_swz(c)] = val[u].y;
+                row[(t0 + 2) ^ lds_swz(c)] = val[u].z;
+                row[(t0 + 3) ^ lds_swz(c)] = val[u].w;
             }
         }
-        lds_barrier();
-        const bool more = tile + 1 < tileEnd;
-        const TileId done = cur;
-        const BlockOrigin od = origin_of(raw, a.g);
-        // NHWC side of the finished tile: LDS -> base tensor; pixels outside the image are dropped
-        // (sparse_gather.cc:121).  The loads of the next tile are issued after these stores (k_gather_planar
-        // says why).
-        if (od.valid) {
-            const uint32_t items = (uint32_t)done.Pn << a.lppLog;
-            for (uint32_t base = 0; base < items; base += nthr * 4) {
-                vec w[4];
-                int64_t dst[4];
+    }
+    lds_barrier();
+
+    // NHWC side: LDS -> base tensor; pixels outside the image are dropped (sparse_gather.cc:121)
+    const BlockOrigin o = origin_of(raw, a.g);
+    if (!o.valid) return;
+    const uint32_t items = (uint32_t)t.Pn << a.lppLog;
+    for (uint32_t base = 0; base < items; base += nthr * 4) {
+        vec w[4];
+        int64_t dst[4];
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    const uint32_t i = base + u * nthr + tid;
-                    dst[u] = -1;
-                    w[u] = vzero<VEC>();
-                    if (i < items) {
-                        const uint32_t pl = i >> a.lppLog, cl = i & lppMask;
-                        const uint32_t p = (uint32_t)done.p0 + pl;
-                        const uint32_t r = fdiv(p, a.dS);
-                        const int hh = od.h0 + (int)r, ww = od.w0 + (int)(p - r * a.g.S);
-                        const int cg = done.c0 + (int)cl * VEC;
-                        if ((unsigned)hh < (unsigned)a.g.H && (unsigned)ww < (unsigned)a.g.W && cg < a.g.C) {
-                            dst[u] = (((int64_t)od.n * a.g.H + hh) * a.g.W + ww) * CV + (cg / VEC);
+        for (int u = 0; u < 4; ++u) {
+            const uint32_t i = base + u * nthr + tid;
+            dst[u] = -1;
+            w[u] = vzero<VEC>();
+            if (i < items) {
+                const uint32_t pl = i >> a.lppLog, cl = i & lppMask;
+                const uint32_t p = (uint32_t)t.p0 + pl;
+                const uint32_t r = fdiv(p, a.dS);
+                const int hh = o.h0 + (int)r, ww = o.w0 + (int)(p - r * a.g.S);
+                const int cg = t.c0 + (int)cl * VEC;
+                if ((unsigned)hh < (unsigned)a.g.H && (unsigned)ww < (unsigned)a.g.W && cg < a.g.C) {
+                    dst[u] = (((int64_t)o.n * a.g.H + hh) * a.g.W + ww) * CV + (cg / VEC);
 #pragma unroll
-                            for (int k = 0; k < VEC; ++k) {
-                                const uint32_t c = cl * VEC + k;
-                                vset(w[u], k, lds[c * a.Pp + (pl ^ lds_swz(c))]);
-                            }
-                        }
+                    for (int k = 0; k < VEC; ++k) {
+                        const uint32_t c = cl * VEC + k;
+                        vset(w[u], k, lds[c * a.Pp + (pl ^ lds_swz(c))]);
                     }
                 }
-                if (MODE == SCATTER_ADD) {
-                    vec curv[4];
-#pragma unroll
-                    for (int u = 0; u < 4; ++u)
-                        if (dst[u] >= 0) curv[u] = ld_stream(yv + dst[u]);
-#pragma unroll
-                    for (int u = 0; u < 4; ++u)
-                        if (dst[u] >= 0) st_stream(yv + dst[u], vadd(curv[u], w[u]));
-                } else {
-#pragma unroll
-                    for (int u = 0; u < 4; ++u)
-                        if (dst[u] >= 0) commit<VEC, MODE>(yv + dst[u], w[u]);
-                }
             }
         }
-        if (!more) break;
-        decode_tile(a, tile + 1, cur);
-        planar_load_tile(x + ((int64_t)cur.ib * a.g.C + cur.c0) * RS + cur.p0, RS, a, cur, tid, nthr, val);
-        lds_barrier();
-        ++tile;
+        if (MODE == SCATTER_ADD) {
+            vec curv[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (dst[u] >= 0) curv[u] = ld_stream(yv + dst[u]);
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (dst[u] >= 0) st_stream(yv + dst[u], vadd(curv[u], w[u]));
+        } else {
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (dst[u] >= 0) commit<VEC, MODE>(yv + dst[u], w[u]);
+        }
     }
 }
 
@@ -1015,9 +970,9 @@ static uint32_t pow2_ceil(uint32_t v)
     return p;
 }
 
-// Optional overrides for experiments: SBNET_TUNE="ct=32,lds=32768,occ=4".
+// Optional overrides for experiments: SBNET_TUNE="ct=32,lds=32768,wg=256".
 struct Tune {
-    int ct = 0, ldsBytes = 0, wg = 0, occ = 0, dbg = 0;
+    int ct = 0, ldsBytes = 0, wg = 0;
 };
 
 static Tune read_tune()
@@ -1029,8 +984,6 @@ static Tune read_tune()
     if ((p = strstr(s, "ct="))) t.ct = atoi(p + 3);
     if ((p = strstr(s, "lds="))) t.ldsBytes = atoi(p + 4);
     if ((p = strstr(s, "wg="))) t.wg = atoi(p + 3);
-    if ((p = strstr(s, "occ="))) t.occ = atoi(p + 4);
-    if ((p = strstr(s, "dbg="))) t.dbg = atoi(p + 4);
     return t;
 }
 
@@ -1116,21 +1069,7 @@ static bool make_nhwc_args(const Geom& g, int numActive, int vec, NhwcArgs& a)
     return true;
 }
 
-// Compute units of the current device (cached per device index; read-only after the first query).
-static int device_cu_count()
-{
-    static int cus[64] = {0};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-    if (cus[dev] == 0) {
-        int n = 0;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-        cus[dev] = n;
-    }
-    return cus[dev];
-}
-
-// Chooses the tile, the workgroup size and the persistent grid of the planar kernels.
+// Chooses the tile and the workgroup size of the planar kernels; the grid is one workgroup per tile.
 static bool make_tile_args(const Geom& g, int numActive, int vec, TileArgs& a, int& threads, size_t& ldsBytes,
                            unsigned& grid)
 {
@@ -1167,7 +1106,6 @@ static bool make_tile_args(const Geom& g, int numActive, int vec, TileArgs& a, i
     a.psplit = (RS + a.P - 1) / a.P;
     a.Pp = (a.P + 31) / 32 * 32;
     a.vpr = (uint32_t)((a.P + 3) / 4);
-    a.dbg = (uint32_t)tune.dbg;
     a.tpb = (uint32_t)(a.psplit * a.cchunks);
     const uint64_t total = (uint64_t)numActive * a.tpb;
     if (total >= (1ull << 31)) return false;
@@ -1178,16 +1116,7 @@ static bool make_tile_args(const Geom& g, int numActive, int vec, TileArgs& a, i
     a.dVpr = make_fastdiv(a.vpr);
     ldsBytes = (size_t)a.Ct * a.Pp * sizeof(float);
     if (ldsBytes > 64 * 1024) return false;
-    // persistent grid: as many workgroups as the device holds at once (LDS, 2048 threads and 32 waves per CU)
-    int perCu = (int)((160 * 1024) / (ldsBytes + 512));
-    const int byThreads = 2048 / threads;
-    if (perCu > byThreads) perCu = byThreads;
-    if (tune.occ > 0 && perCu > tune.occ) perCu = tune.occ;
-    if (perCu < 1) perCu = 1;
-    const uint64_t slots = (uint64_t)device_cu_count() * perCu;
-    a.tilesPerWg = (uint32_t)((total + slots - 1) / slots);
-    if (a.tilesPerWg < 1) a.tilesPerWg = 1;
-    grid = (unsigned)((total + a.tilesPerWg - 1) / a.tilesPerWg);
+    grid = a.total;
     return true;
 }
 
