@@ -343,6 +343,13 @@ __device__ __forceinline__ void lds_barrier()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
+// 16-byte LDS read of 4 consecutive floats.  The promise of alignment has to be explicit: a plain vector
+// load through a cast pointer was lowered to two 8-byte-pair reads, which serialise on the LDS banks.
+__device__ __forceinline__ f4 lds_read4(const float* p)
+{
+    return *static_cast<const f4*>(__builtin_assume_aligned(p, 16));
+}
+
 // Raw buffer access (V# descriptors): 32-bit byte offsets from a wave-uniform base, and hardware range
 // checking: a load whose offset is outside the descriptor returns 0, a store is dropped.  Lanes with
 // nothing to do get the offset 0xFFFFFFFF instead of a branch, and the addressing needs no 64-bit
@@ -465,7 +472,7 @@ __global__ __launch_bounds__(512) void k_gather_planar(const float* __restrict__
             const uint32_t c = fdiv(i, a.dVpr);
             const uint32_t e0 = 4u * (i - c * a.vpr);
             const bool full = i < slots && e0 + 4u <= (uint32_t)t.Pn;
-            q[u] = *reinterpret_cast<const f4*>(lds + (full ? c * a.Pp + (e0 ^ lds_swz(c)) : 0u));
+            q[u] = lds_read4(lds + (full ? c * a.Pp + (e0 ^ lds_swz(c)) : 0u));
             off[u] = full ? (c * RS + e0) * 4u : BUF_OOB;
         }
 #pragma unroll
@@ -475,7 +482,7 @@ __global__ __launch_bounds__(512) void k_gather_planar(const float* __restrict__
     const uint32_t tail = (uint32_t)t.Pn & 3u;
     if (tail && tid < (uint32_t)t.ctEff) {
         const uint32_t e0 = (uint32_t)t.Pn - tail;
-        const f4 q = *reinterpret_cast<const f4*>(lds + tid * a.Pp + (e0 ^ lds_swz(tid)));
+        const f4 q = lds_read4(lds + tid * a.Pp + (e0 ^ lds_swz(tid)));
         const uint32_t off = (tid * RS + e0) * 4u;
         buf_store<0>(yr, off, q.x);
         if (tail > 1) buf_store<0>(yr, off + 4u, q.y);
