@@ -490,6 +490,162 @@ __global__ __launch_bounds__(512) void k_gather_planar(const float* __restrict__
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Planar gather whose workgroups own whole 128-byte lines of the output
+// ---------------------------------------------------------------------------------------------
+//
+// A write-only probe of the tile pattern above (32 runs of 243 floats at 729-float pitch, 4-byte
+// aligned, first and last line of every run shared with another workgroup) reaches 3.5 TB/s; the same
+// bytes written as whole, 16-byte aligned lines that belong to one workgroup each reach 5.9 TB/s.
+// So this kernel cuts the output differently.  The Ct planes of a channel chunk are one contiguous
+// piece of y, "the chunk", addressed by a linear float index l = c*RS + p.  Tile (chunk, split) still
+// reads the pixels [p0, p1) for all Ct channels, but for row c it writes the lines that START inside
+// [c*RS + p0, c*RS + p1): the range [up(c*RS + p0), up(c*RS + p1)), up() rounding to the next line of
+// y (the two ends of the chunk stay where they are).  These ranges tile the chunk exactly, every store
+// is an aligned dwordx4, and no line is written by two workgroups (except the one line two chunks may
+// share).  The price is that a tile needs up to 31 pixels beyond p1 -- for the last split of a plane,
+// where row c's last line runs into row c+1, the first 31 pixels of the plane -- so the tile's pixel
+// window is [p0, p1 + LINE_EXT) taken cyclically over the plane, about 13 % more NHWC reads at 243
+// pixels per tile.  Reads were never the problem (the same NHWC read pattern alone runs at 6.6 TB/s).
+//
+// LDS: row c at c*Pp, window pixel q at column q + phi(c), phi(c) = (c*RS + p0) & 3, XOR-swizzled as
+// above.  The shift phi makes LDS columns congruent to l modulo 4, so an output slot that lies inside
+// one row is one ds_read_b128.  Slots that cross into the next row (up to 9 per row, and only in the
+// last split) are assembled from four 4-byte reads.
+
+constexpr int LINE_FLOATS = 32;
+constexpr int LINE_EXT = LINE_FLOATS - 1;
+
+struct LineArgs {
+    Geom g;
+    int Ct, lppLog;
+    int RS;
+    int P, Pp, psplit, cchunks;
+    int ext;            // window pixels beyond the tile's own: LINE_EXT, or 0 when a tile takes whole planes
+    int xcd;            // > 0: tiles of one chunk are spread over workgroup ids xcd apart
+    uint32_t tpb, total;
+    uint32_t spr;       // bound on the output slots of one row of one tile
+    int64_t imgFloats;
+    uint32_t imgBytes;
+    FastDiv dTpb, dPs, dS, dSpr, dRS;
+};
+
+template <int LD>
+__global__ __launch_bounds__(512) void k_gather_lines(const float* __restrict__ x, float* __restrict__ y,
+                                                      const int16_t* __restrict__ idx, LineArgs a)
+{
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const uint32_t tid = threadIdx.x, nthr = blockDim.x;
+    const uint32_t RS = (uint32_t)a.RS;
+
+    // tile id.  Consecutive workgroup ids go to different XCDs (each with its own L2); with xcd set, the
+    // splits of one chunk, whose windows overlap, get ids that are xcd apart and so share an L2.
+    uint32_t id = blockIdx.x;
+    if (a.xcd > 0) {
+        const uint32_t group = (uint32_t)a.xcd * (uint32_t)a.psplit;
+        const uint32_t full = a.total / group * group;
+        if (id < full) {
+            const uint32_t gidx = id / group, r = id - gidx * group;
+            const uint32_t lane = r % (uint32_t)a.xcd, split = r / (uint32_t)a.xcd;
+            id = (gidx * (uint32_t)a.xcd + lane) * (uint32_t)a.psplit + split;
+        }
+    }
+    const uint32_t ib = fdiv(id, a.dTpb);
+    const uint32_t rem = id - ib * a.tpb;
+    const uint32_t cc = fdiv(rem, a.dPs);
+    const uint32_t split = rem - cc * (uint32_t)a.psplit;
+    const uint32_t c0 = cc * (uint32_t)a.Ct;
+    const uint32_t ctEff = min((uint32_t)a.Ct, (uint32_t)a.g.C - c0);
+    const uint32_t p0 = split * (uint32_t)a.P;
+    const uint32_t p1 = min(p0 + (uint32_t)a.P, RS);
+    const uint32_t win = p1 - p0 + (uint32_t)a.ext;
+
+    const BlockOrigin o = origin_of(load_triple(idx, ib), a.g);
+    const rsrc_t xr = make_rsrc(x + (o.valid ? (int64_t)o.n * a.imgFloats : 0), o.valid ? a.imgBytes : 0u);
+
+    // NHWC side: lane owns channels [4*cl, 4*cl + 4) of window pixels q0 + u*step
+    const uint32_t cl = tid & ((1u << a.lppLog) - 1u);
+    const uint32_t q0 = tid >> a.lppLog, step = nthr >> a.lppLog;
+    const uint32_t c = c0 + cl * 4u;
+    const bool cok = c < (uint32_t)a.g.C;
+    f4 v[LD];
+#pragma unroll
+    for (int u = 0; u < LD; ++u) {
+        const uint32_t q = q0 + (uint32_t)u * step;
+        uint32_t p = p0 + q;
+        if (p >= RS) p -= RS;  // the window wraps to the start of the plane
+        const uint32_t r = fdiv(p, a.dS), sc = p - r * (uint32_t)a.g.S;
+        const int hh = o.h0 + (int)r, ww = o.w0 + (int)sc;
+        const bool ok = cok && q < win && (unsigned)hh < (unsigned)a.g.H && (unsigned)ww < (unsigned)a.g.W;
+        const uint32_t off = (((uint32_t)hh * (uint32_t)a.g.W + (uint32_t)ww) * (uint32_t)a.g.C + c) * 4u;
+        v[u] = buf_load<4>(xr, ok ? off : BUF_OOB);
+    }
+#pragma unroll
+    for (int u = 0; u < LD; ++u) {
+        const uint32_t q = q0 + (uint32_t)u * step;
+        if (q < win) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t cr = cl * 4u + (uint32_t)k;
+                const uint32_t phi = ((uint32_t)k * RS + p0) & 3u;  // == (cr*RS + p0) & 3
+                lds[cr * (uint32_t)a.Pp + ((q + phi) ^ lds_swz(cr))] = vget(v[u], k);
+            }
+        }
+    }
+    lds_barrier();
+
+    // planar side: whole lines of the chunk
+    const int64_t chunkBase = ((int64_t)ib * a.g.C + c0) * RS;
+    const uint32_t chunkFloats = ctEff * RS;
+    const uint32_t a0 = (uint32_t)(((reinterpret_cast<uintptr_t>(y) >> 2) + (uint64_t)chunkBase) & (LINE_FLOATS - 1));
+    const rsrc_t yr = make_rsrc(y + chunkBase, chunkFloats * 4u);
+    // a tile that takes whole planes owns the whole chunk: its slots are simply l = 0, 4, 8, ...
+    const bool whole = a.psplit == 1;
+    const uint32_t slots = whole ? chunkFloats >> 2 : ctEff * a.spr;
+    for (uint32_t base = 0; base < slots; base += 4 * nthr) {
+        f4 qv[4];
+        uint32_t off[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const uint32_t i = base + (uint32_t)u * nthr + tid;
+            uint32_t cr, l;
+            bool live = i < slots;
+            if (whole) {
+                l = 4u * i;
+                cr = fdiv(l, a.dRS);
+            } else {
+                cr = fdiv(i, a.dSpr);
+                const uint32_t k = i - cr * a.spr;
+                const uint32_t lin0 = cr * RS + p0, lin1 = cr * RS + p1;
+                const uint32_t A = (lin0 == 0) ? 0u : ((a0 + lin0 + LINE_EXT) & ~(uint32_t)LINE_EXT) - a0;
+                const uint32_t B =
+                    (lin1 == chunkFloats) ? chunkFloats : ((a0 + lin1 + LINE_EXT) & ~(uint32_t)LINE_EXT) - a0;
+                l = A + 4u * k;
+                live = live && l < B;
+            }
+            const uint32_t lin0 = cr * RS + p0;
+            const bool inrow = l + 4u <= (cr + 1u) * RS;
+            const uint32_t col = l - lin0 + (lin0 & 3u);
+            qv[u] = lds_read4(lds + ((live && inrow) ? cr * (uint32_t)a.Pp + (col ^ lds_swz(cr)) : 0u));
+            if (live && !inrow) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const uint32_t le = l + (uint32_t)e;
+                    const uint32_t ce = fdiv(le, a.dRS);  // planes shorter than a line can be crossed twice
+                    const uint32_t pe = le - ce * RS;     // pixel inside plane ce
+                    uint32_t qe = pe - p0;                // its place in the cyclic window
+                    if (pe < p0) qe += RS;
+                    const uint32_t phi = (ce * RS + p0) & 3u;
+                    vset(qv[u], e, lds[ce * (uint32_t)a.Pp + ((qe + phi) ^ lds_swz(ce))]);
+                }
+            }
+            off[u] = live ? l * 4u : BUF_OOB;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) buf_store<BUF_NT>(yr, off[u], qv[u]);
+    }
+}
+
 // sparse_gather.cc:103-130 with transpose == true: the block stack is [blocks, C, R, S].
 template <int VEC, int MODE>
 __global__ __launch_bounds__(512) void k_scatter_planar(const float* __restrict__ x, float* __restrict__ y,
@@ -1001,9 +1157,9 @@ static uint32_t pow2_ceil(uint32_t v)
     return p;
 }
 
-// Optional overrides for experiments: SBNET_TUNE="ct=32,lds=32768,wg=256".
+// Optional overrides for experiments: SBNET_TUNE="ct=32,lds=32768,wg=256,ps=3,xcd=8,lines=1".
 struct Tune {
-    int ct = 0, ldsBytes = 0, wg = 0;
+    int ct = 0, ldsBytes = 0, wg = 0, ps = 0, xcd = -1, lines = -1;
 };
 
 static Tune read_tune()
@@ -1015,6 +1171,9 @@ static Tune read_tune()
     if ((p = strstr(s, "ct="))) t.ct = atoi(p + 3);
     if ((p = strstr(s, "lds="))) t.ldsBytes = atoi(p + 4);
     if ((p = strstr(s, "wg="))) t.wg = atoi(p + 3);
+    if ((p = strstr(s, "ps="))) t.ps = atoi(p + 3);
+    if ((p = strstr(s, "xcd="))) t.xcd = atoi(p + 4);
+    if ((p = strstr(s, "lines="))) t.lines = atoi(p + 6);
     return t;
 }
 
@@ -1154,6 +1313,72 @@ static bool make_tile_args(const Geom& g, int numActive, int vec, TileArgs& a, i
     return true;
 }
 
+// Tile choice of k_gather_lines.  Returns false where the kernel does not apply (the caller then uses
+// k_gather_planar): y not 16-byte aligned, a last split shorter than the window extension, LDS.
+static bool make_line_args(const Geom& g, int numActive, const float* y, LineArgs& a, int& threads, int& ld,
+                           size_t& ldsBytes, unsigned& grid)
+{
+    static const Tune tune = read_tune();
+    if (tune.lines == 0) return false;
+    if (g.C % 4 != 0 || (reinterpret_cast<uintptr_t>(y) & 15) != 0) return false;
+    a.g = g;
+    const int64_t RS64 = (int64_t)g.R * g.S;
+    a.imgFloats = (int64_t)g.H * g.W * g.C;
+    if (RS64 < 4 || a.imgFloats >= (1ll << 30) || (int64_t)g.C * RS64 >= (1ll << 30)) return false;
+    const int RS = (int)RS64;
+    a.RS = RS;
+    a.imgBytes = (uint32_t)(a.imgFloats * 4);
+    int lpp = 1;
+    while (lpp * 2 * 4 <= 32 && lpp * 4 < g.C) lpp *= 2;
+    a.Ct = lpp * 4;
+    a.lppLog = ilog2_floor((uint32_t)lpp);
+    a.cchunks = (g.C + a.Ct - 1) / a.Ct;
+    // The smallest workgroup whose LD vectors per thread cover a whole plane; otherwise 512 threads and as
+    // few splits as the window (own pixels + LINE_EXT) allows within 5 vectors per thread.
+    const int maxLd = 5;
+    threads = 0;
+    a.psplit = 1;
+    for (int nthr = 64; nthr <= 512; nthr *= 2) {
+        threads = nthr;
+        if (4 * nthr / lpp >= RS) break;
+    }
+    if (4 * threads / lpp < RS) {
+        const int cap = maxLd * threads / lpp - LINE_EXT;
+        if (cap < 2 * LINE_FLOATS) return false;
+        a.psplit = (RS + cap - 1) / cap;
+    }
+    if (tune.ps > 0) a.psplit = tune.ps;
+    a.P = (RS + a.psplit - 1) / a.psplit;
+    a.psplit = (RS + a.P - 1) / a.P;
+    a.ext = a.psplit > 1 ? LINE_EXT : 0;
+    if (a.psplit > 1 && RS - (a.psplit - 1) * a.P < LINE_FLOATS) return false;  // last split must hold the extension
+    const int win = a.P + a.ext;
+    ld = (win * lpp + threads - 1) / threads;
+    if (ld < 4) ld = 4;
+    if (ld > 8) return false;
+    a.Pp = (win + 3 + 31) / 32 * 32;
+    ldsBytes = (size_t)a.Ct * a.Pp * sizeof(float);
+    if (ldsBytes > 64 * 1024) return false;
+    // slots per row: the written range of a row is at most P + LINE_EXT floats; when every chunk starts on a
+    // line it is a whole number of lines
+    const bool aligned = (reinterpret_cast<uintptr_t>(y) & 127) == 0 && ((int64_t)a.Ct * RS) % LINE_FLOATS == 0 &&
+                         ((int64_t)g.C * RS) % LINE_FLOATS == 0;
+    a.spr = aligned ? (uint32_t)((a.P + LINE_EXT) / LINE_FLOATS * (LINE_FLOATS / 4)) : (uint32_t)((a.P + LINE_EXT + 3) / 4);
+    if (a.psplit == 1) a.spr = 1;  // unused: such a tile enumerates the chunk's slots directly
+    a.tpb = (uint32_t)(a.psplit * a.cchunks);
+    const uint64_t total = (uint64_t)numActive * a.tpb;
+    if (total >= (1ull << 31)) return false;
+    a.total = (uint32_t)total;
+    a.xcd = tune.xcd >= 0 ? tune.xcd : 0;
+    a.dTpb = make_fastdiv(a.tpb);
+    a.dPs = make_fastdiv((uint32_t)a.psplit);
+    a.dS = make_fastdiv((uint32_t)g.S);
+    a.dSpr = make_fastdiv(a.spr);
+    a.dRS = make_fastdiv((uint32_t)RS);
+    grid = a.total;
+    return true;
+}
+
 template <int VEC>
 static void gather_dispatch(const float* x, float* y, const int16_t* idx, const Geom& g, int numActive,
                             bool transpose, hipStream_t stream, hipError_t& err)
@@ -1167,6 +1392,20 @@ static void gather_dispatch(const float* x, float* y, const int16_t* idx, const 
         int threads;
         size_t lds;
         unsigned grid;
+        if (VEC == 4) {
+            LineArgs la;
+            int ld;
+            if (make_line_args(g, numActive, y, la, threads, ld, lds, grid)) {
+                switch (ld) {
+                case 4: hipLaunchKernelGGL(k_gather_lines<4>, dim3(grid), dim3(threads), lds, stream, x, y, idx, la); break;
+                case 5: hipLaunchKernelGGL(k_gather_lines<5>, dim3(grid), dim3(threads), lds, stream, x, y, idx, la); break;
+                case 6: hipLaunchKernelGGL(k_gather_lines<6>, dim3(grid), dim3(threads), lds, stream, x, y, idx, la); break;
+                case 7: hipLaunchKernelGGL(k_gather_lines<7>, dim3(grid), dim3(threads), lds, stream, x, y, idx, la); break;
+                default: hipLaunchKernelGGL(k_gather_lines<8>, dim3(grid), dim3(threads), lds, stream, x, y, idx, la); break;
+                }
+                return;
+            }
+        }
         // 32 KB tiles: 46.5 us against 52.7 us with 16 KB tiles on the 800x800x128 workload.
         // Planes of fewer than 4 pixels and images or blocks beyond 32-bit byte offsets take the generic kernel.
         if ((int64_t)g.R * g.S < 4 || !make_tile_args(g, numActive, VEC, a, threads, lds, grid, 32 * 1024)) {

@@ -264,6 +264,51 @@ def test_misaligned_base_pointers():
             assert float(ybuf[:off].min()) == 10.0 and float(ybuf[off + x.size:].max()) == 10.0
 
 
+@pytest.mark.parametrize("geom", [
+    # (H, W, C), bsize, bstride, boffset, out offset in floats, N
+    ((120, 130, 128), (27, 27), (25, 25), (-1, -1), 0, 1),    # 3 splits per plane, chunks start on 128-byte lines
+    ((120, 130, 128), (27, 27), (25, 25), (-1, -1), 4, 1),    # same, output 16 bytes past a line
+    ((120, 130, 128), (27, 27), (25, 25), (-1, -1), 20, 2),   # 80 bytes past a line
+    ((120, 130, 20), (27, 27), (25, 25), (-1, -1), 0, 1),     # one partial chunk (20 of 32 channels), odd chunk starts
+    ((120, 130, 48), (27, 27), (25, 25), (-1, -1), 8, 2),     # full chunk + partial chunk
+    ((100, 90, 16), (21, 23), (20, 20), (-3, -2), 0, 1),      # 483-pixel planes, 2 splits, 16-channel chunks
+    ((100, 90, 36), (19, 17), (19, 17), (0, 0), 12, 1),       # 323-pixel planes
+    ((64, 64, 8), (5, 5), (5, 5), (0, 0), 0, 3),              # planes shorter than a line: a line crosses two planes
+    ((64, 64, 8), (5, 5), (5, 5), (0, 0), 28, 3),
+    ((64, 64, 32), (3, 3), (2, 2), (-1, -1), 0, 1),           # 9-pixel planes
+    ((64, 64, 4), (9, 7), (9, 7), (0, 0), 4, 2),              # single 4-channel vector per pixel
+    ((300, 300, 32), (32, 32), (32, 32), (0, 0), 0, 1),       # planes that are whole lines, 5 splits
+    ((300, 300, 32), (33, 31), (30, 30), (-2, -2), 16, 1),
+])
+def test_planar_gather_owns_whole_lines(geom):
+    """Planar gather into outputs at every kind of alignment against 128-byte lines: the kernel assigns whole
+    lines of the stack to workgroups, so chunk starts, split points and plane ends that fall inside a line are
+    the cases to cover; guard zones around the output must stay untouched."""
+    (H, W, C), bs, bst, bo, off, N = geom
+    rng = np.random.default_rng(H * 7 + C + off)
+    bc = bcount_covering(H, W, bst, bo)
+    x = rng.standard_normal((N, H, W, C)).astype(np.float32)
+    cells = rng.random((N, bc[0], bc[1])) < 0.6
+    cells[0, 0, 0] = cells[-1, -1, -1] = True
+    idx = np.ascontiguousarray(np.argwhere(cells), dtype=np.int16)
+    rng.shuffle(idx, axis=0)  # the op takes any list order
+    cnt = np.array([idx.shape[0]], dtype=np.int32)
+    g_o = orc.sparse_gather(x, cnt, idx, bs, bst, bo, transpose=True)
+    guard = 64
+    gbuf = torch.full((g_o.size + off + 2 * guard,), 777.0, dtype=torch.float32, device=DEV)
+    assert gbuf.data_ptr() % 128 == 0
+    gout = gbuf[guard + off:guard + off + g_o.size].view(*g_o.shape)
+    sbnet_amd.sparse_gather(dev(x), cnt, dev(idx), bs, bst, bo, transpose=True, out=gout)
+    np.testing.assert_array_equal(host(gout), g_o)
+    assert float(gbuf[:guard + off].min()) == 777.0 and float(gbuf[:guard + off].max()) == 777.0
+    assert float(gbuf[guard + off + g_o.size:].min()) == 777.0 and float(gbuf[guard + off + g_o.size:].max()) == 777.0
+    # and back: the planar scatter restores exactly the gathered pixels
+    yd = torch.zeros((N, H, W, C), dtype=torch.float32, device=DEV)
+    sbnet_amd.sparse_scatter_var(gout, cnt, dev(idx), yd, bs, bst, bo, add=False, transpose=True)
+    y_o = orc.sparse_scatter(g_o, cnt, idx, np.zeros_like(x), bs, bst, bo, add=False, transpose=True)
+    np.testing.assert_array_equal(host(yd), y_o)
+
+
 # ---------------------------------------------------------------------------------------------
 # reduce_mask: summation order, thresholds, sizes
 # ---------------------------------------------------------------------------------------------
