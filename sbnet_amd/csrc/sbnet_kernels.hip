@@ -133,7 +133,11 @@ __device__ __forceinline__ RawTriple load_triple(const int16_t* __restrict__ idx
 {
     const uint32_t byteOff = 6u * (uint32_t)__builtin_amdgcn_readfirstlane(ib);
     const uintptr_t base = reinterpret_cast<uintptr_t>(idx) + byteOff;
-    const uint32_t* __restrict__ w = reinterpret_cast<const uint32_t*>(base & ~(uintptr_t)3);
+    // constant address space: a uniform address alone does not make the compiler pick a scalar load, and a
+    // triple that arrives in vector registers makes every descriptor built from it "divergent" (each buffer
+    // access then sits in a readfirstlane loop).  The list is never written by the kernels that read it.
+    typedef const uint32_t __attribute__((address_space(4))) * const_u32_ptr;
+    const_u32_ptr w = (const_u32_ptr)(base & ~(uintptr_t)3);
     RawTriple r;
     r.lo = w[0];
     r.hi = w[1];
@@ -563,32 +567,65 @@ __global__ __launch_bounds__(512) void k_gather_lines(const float* __restrict__ 
     const BlockOrigin o = origin_of(load_triple(idx, ib), a.g);
     const rsrc_t xr = make_rsrc(x + (o.valid ? (int64_t)o.n * a.imgFloats : 0), o.valid ? a.imgBytes : 0u);
 
-    // NHWC side: lane owns channels [4*cl, 4*cl + 4) of window pixels q0 + u*step
+    // NHWC side: lane owns channels [4*cl, 4*cl + 4) of window pixels q0 + u*step.  (r, s) of the pixel is
+    // kept by increments; stepping past the end of the plane wraps to its start, which is r -= R.
     const uint32_t cl = tid & ((1u << a.lppLog) - 1u);
     const uint32_t q0 = tid >> a.lppLog, step = nthr >> a.lppLog;
     const uint32_t c = c0 + cl * 4u;
     const bool cok = c < (uint32_t)a.g.C;
+    const uint32_t stepR = fdiv(step, a.dS), stepS = step - stepR * (uint32_t)a.g.S;
+    uint32_t r, sc;
+    {
+        uint32_t p = p0 + q0;
+        if (p >= RS) p -= RS;
+        r = fdiv(p, a.dS);
+        sc = p - r * (uint32_t)a.g.S;
+    }
     f4 v[LD];
 #pragma unroll
     for (int u = 0; u < LD; ++u) {
         const uint32_t q = q0 + (uint32_t)u * step;
-        uint32_t p = p0 + q;
-        if (p >= RS) p -= RS;  // the window wraps to the start of the plane
-        const uint32_t r = fdiv(p, a.dS), sc = p - r * (uint32_t)a.g.S;
         const int hh = o.h0 + (int)r, ww = o.w0 + (int)sc;
         const bool ok = cok && q < win && (unsigned)hh < (unsigned)a.g.H && (unsigned)ww < (unsigned)a.g.W;
         const uint32_t off = (((uint32_t)hh * (uint32_t)a.g.W + (uint32_t)ww) * (uint32_t)a.g.C + c) * 4u;
         v[u] = buf_load<4>(xr, ok ? off : BUF_OOB);
+        sc += stepS;
+        r += stepR;
+        if (sc >= (uint32_t)a.g.S) {
+            sc -= (uint32_t)a.g.S;
+            ++r;
+        }
+        if (r >= (uint32_t)a.g.R) r -= (uint32_t)a.g.R;
     }
+    // registers -> LDS.  With a pixel step that is a multiple of 32 the swizzle (bits 2..4 of the column) does
+    // not depend on u, and the column of (u, k) is the column of (0, k) plus u*step.
+    {
+        const uint32_t swz = lds_swz(cl * 4u);
+        uint32_t rowAddr[4];
 #pragma unroll
-    for (int u = 0; u < LD; ++u) {
-        const uint32_t q = q0 + (uint32_t)u * step;
-        if (q < win) {
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t phi = ((uint32_t)k * RS + p0) & 3u;  // == ((4*cl + k)*RS + p0) & 3
+            rowAddr[k] = (cl * 4u + (uint32_t)k) * (uint32_t)a.Pp + phi;
+        }
+        if ((step & 31u) == 0) {
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const uint32_t cr = cl * 4u + (uint32_t)k;
-                const uint32_t phi = ((uint32_t)k * RS + p0) & 3u;  // == (cr*RS + p0) & 3
-                lds[cr * (uint32_t)a.Pp + ((q + phi) ^ lds_swz(cr))] = vget(v[u], k);
+            for (int k = 0; k < 4; ++k) rowAddr[k] = (rowAddr[k] & ~3u) + (((rowAddr[k] & 3u) + q0) ^ swz);
+#pragma unroll
+            for (int u = 0; u < LD; ++u) {
+                if (q0 + (uint32_t)u * step < win) {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) lds[rowAddr[k] + (uint32_t)u * step] = vget(v[u], k);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < LD; ++u) {
+                const uint32_t q = q0 + (uint32_t)u * step;
+                if (q < win) {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k)
+                        lds[(rowAddr[k] & ~3u) + (((rowAddr[k] & 3u) + q) ^ swz)] = vget(v[u], k);
+                }
             }
         }
     }
@@ -599,50 +636,79 @@ __global__ __launch_bounds__(512) void k_gather_lines(const float* __restrict__ 
     const uint32_t chunkFloats = ctEff * RS;
     const uint32_t a0 = (uint32_t)(((reinterpret_cast<uintptr_t>(y) >> 2) + (uint64_t)chunkBase) & (LINE_FLOATS - 1));
     const rsrc_t yr = make_rsrc(y + chunkBase, chunkFloats * 4u);
-    // a tile that takes whole planes owns the whole chunk: its slots are simply l = 0, 4, 8, ...
-    const bool whole = a.psplit == 1;
-    const uint32_t slots = whole ? chunkFloats >> 2 : ctEff * a.spr;
-    for (uint32_t base = 0; base < slots; base += 4 * nthr) {
-        f4 qv[4];
-        uint32_t off[4];
+    if (a.psplit == 1) {
+        // a tile that takes whole planes owns the whole chunk: its slots are simply l = 0, 4, 8, ...
+        const uint32_t slots = chunkFloats >> 2;
+        for (uint32_t base = 0; base < slots; base += 4 * nthr) {
+            f4 qv[4];
+            uint32_t off[4];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const uint32_t i = base + (uint32_t)u * nthr + tid;
-            uint32_t cr, l;
-            bool live = i < slots;
-            if (whole) {
-                l = 4u * i;
-                cr = fdiv(l, a.dRS);
-            } else {
-                cr = fdiv(i, a.dSpr);
-                const uint32_t k = i - cr * a.spr;
-                const uint32_t lin0 = cr * RS + p0, lin1 = cr * RS + p1;
-                const uint32_t A = (lin0 == 0) ? 0u : ((a0 + lin0 + LINE_EXT) & ~(uint32_t)LINE_EXT) - a0;
-                const uint32_t B =
-                    (lin1 == chunkFloats) ? chunkFloats : ((a0 + lin1 + LINE_EXT) & ~(uint32_t)LINE_EXT) - a0;
-                l = A + 4u * k;
-                live = live && l < B;
-            }
-            const uint32_t lin0 = cr * RS + p0;
-            const bool inrow = l + 4u <= (cr + 1u) * RS;
-            const uint32_t col = l - lin0 + (lin0 & 3u);
-            qv[u] = lds_read4(lds + ((live && inrow) ? cr * (uint32_t)a.Pp + (col ^ lds_swz(cr)) : 0u));
-            if (live && !inrow) {
+            for (int u = 0; u < 4; ++u) {
+                const uint32_t i = base + (uint32_t)u * nthr + tid;
+                const uint32_t l = 4u * i;
+                const uint32_t cr = fdiv(l, a.dRS);
+                const bool live = i < slots;
+                const uint32_t lin0 = cr * RS;
+                const bool inrow = l + 4u <= lin0 + RS;
+                const uint32_t col = l - lin0 + (lin0 & 3u);
+                qv[u] = lds_read4(lds + ((live && inrow) ? cr * (uint32_t)a.Pp + (col ^ lds_swz(cr)) : 0u));
+                if (live && !inrow) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const uint32_t le = l + (uint32_t)e;
-                    const uint32_t ce = fdiv(le, a.dRS);  // planes shorter than a line can be crossed twice
-                    const uint32_t pe = le - ce * RS;     // pixel inside plane ce
-                    uint32_t qe = pe - p0;                // its place in the cyclic window
-                    if (pe < p0) qe += RS;
-                    const uint32_t phi = (ce * RS + p0) & 3u;
-                    vset(qv[u], e, lds[ce * (uint32_t)a.Pp + ((qe + phi) ^ lds_swz(ce))]);
+                    for (int e = 0; e < 4; ++e) {
+                        const uint32_t le = l + (uint32_t)e;
+                        const uint32_t ce = fdiv(le, a.dRS);  // planes shorter than a slot pitch can be crossed twice
+                        const uint32_t pe = le - ce * RS;
+                        vset(qv[u], e, lds[ce * (uint32_t)a.Pp + ((pe + ((ce * RS) & 3u)) ^ lds_swz(ce))]);
+                    }
                 }
+                off[u] = live ? l * 4u : BUF_OOB;
             }
-            off[u] = live ? l * 4u : BUF_OOB;
-        }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) buf_store<BUF_NT>(yr, off[u], qv[u]);
+            for (int u = 0; u < 4; ++u) buf_store<BUF_NT>(yr, off[u], qv[u]);
+        }
+    } else {
+        // One wave per row, four rows in flight: everything about the row (its range [A, B) of whole lines,
+        // where it ends, its swizzle) is wave-uniform and stays on the scalar unit; a lane only adds 4*k.
+        const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+        const uint32_t lane = tid & 63u, nwaves = nthr >> 6;
+        for (uint32_t cr0 = wave; cr0 < ctEff; cr0 += 4u * nwaves) {
+            for (uint32_t kb = 0; kb < a.spr; kb += 64u) {
+                f4 qv[4];
+                uint32_t off[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const uint32_t cr = cr0 + (uint32_t)u * nwaves;
+                    const uint32_t lin0 = cr * RS + p0, lin1 = cr * RS + p1;
+                    const uint32_t A = (lin0 == 0) ? 0u : ((a0 + lin0 + LINE_EXT) & ~(uint32_t)LINE_EXT) - a0;
+                    const uint32_t B = (cr >= ctEff)          ? 0u
+                                       : (lin1 == chunkFloats) ? chunkFloats
+                                                               : ((a0 + lin1 + LINE_EXT) & ~(uint32_t)LINE_EXT) - a0;
+                    const uint32_t rowEnd = lin0 - p0 + RS;
+                    const uint32_t colBase = A - lin0 + (lin0 & 3u);  // multiple of 4 less than 36
+                    const uint32_t k4 = 4u * (kb + lane);
+                    const uint32_t l = A + k4;
+                    const bool live = l < B;
+                    const bool inrow = l + 4u <= rowEnd;
+                    qv[u] = lds_read4(lds + ((live && inrow) ? cr * (uint32_t)a.Pp + ((colBase + k4) ^ lds_swz(cr)) : 0u));
+                    if (live && !inrow) {
+                        // only in the last split: the row's last line runs into the first pixels of the next plane,
+                        // which sit at the end of the cyclic window
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const uint32_t le = l + (uint32_t)e;
+                            const uint32_t ce = le >= rowEnd ? cr + 1u : cr;  // RS > LINE_EXT here: one crossing at most
+                            const uint32_t pe = le - ce * RS;
+                            const uint32_t qe = pe < p0 ? pe + RS - p0 : pe - p0;
+                            const uint32_t phi = (ce * RS + p0) & 3u;
+                            vset(qv[u], e, lds[ce * (uint32_t)a.Pp + ((qe + phi) ^ lds_swz(ce))]);
+                        }
+                    }
+                    off[u] = live ? l * 4u : BUF_OOB;
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) buf_store<BUF_NT>(yr, off[u], qv[u]);
+            }
+        }
     }
 }
 
