@@ -510,7 +510,9 @@ __global__ __launch_bounds__(512) void k_gather_planar(const float* __restrict__
 // share).  The price is that a tile needs up to 31 pixels beyond p1 -- for the last split of a plane,
 // where row c's last line runs into row c+1, the first 31 pixels of the plane -- so the tile's pixel
 // window is [p0, p1 + LINE_EXT) taken cyclically over the plane, about 13 % more NHWC reads at 243
-// pixels per tile.  Reads were never the problem (the same NHWC read pattern alone runs at 6.6 TB/s).
+// pixels per tile; the extra pixels are read by the neighbouring tile as well and come from cache (a
+// bare read-and-write of this access pattern takes the same time with and without them).  Used when a
+// plane is split over several tiles; a tile of whole planes already writes one contiguous piece.
 //
 // LDS: row c at c*Pp, window pixel q at column q + phi(c), phi(c) = (c*RS + p0) & 3, XOR-swizzled as
 // above.  The shift phi makes LDS columns congruent to l modulo 4, so an output slot that lies inside
@@ -525,13 +527,13 @@ struct LineArgs {
     int Ct, lppLog;
     int RS;
     int P, Pp, psplit, cchunks;
-    int ext;            // window pixels beyond the tile's own: LINE_EXT, or 0 when a tile takes whole planes
+    int ext;            // window pixels beyond the tile's own: LINE_EXT
     int xcd;            // > 0: tiles of one chunk are spread over workgroup ids xcd apart
     uint32_t tpb, total;
     uint32_t spr;       // bound on the output slots of one row of one tile
     int64_t imgFloats;
     uint32_t imgBytes;
-    FastDiv dTpb, dPs, dS, dSpr, dRS;
+    FastDiv dTpb, dPs, dS;
 };
 
 template <int LD>
@@ -636,37 +638,7 @@ __global__ __launch_bounds__(512) void k_gather_lines(const float* __restrict__ 
     const uint32_t chunkFloats = ctEff * RS;
     const uint32_t a0 = (uint32_t)(((reinterpret_cast<uintptr_t>(y) >> 2) + (uint64_t)chunkBase) & (LINE_FLOATS - 1));
     const rsrc_t yr = make_rsrc(y + chunkBase, chunkFloats * 4u);
-    if (a.psplit == 1) {
-        // a tile that takes whole planes owns the whole chunk: its slots are simply l = 0, 4, 8, ...
-        const uint32_t slots = chunkFloats >> 2;
-        for (uint32_t base = 0; base < slots; base += 4 * nthr) {
-            f4 qv[4];
-            uint32_t off[4];
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const uint32_t i = base + (uint32_t)u * nthr + tid;
-                const uint32_t l = 4u * i;
-                const uint32_t cr = fdiv(l, a.dRS);
-                const bool live = i < slots;
-                const uint32_t lin0 = cr * RS;
-                const bool inrow = l + 4u <= lin0 + RS;
-                const uint32_t col = l - lin0 + (lin0 & 3u);
-                qv[u] = lds_read4(lds + ((live && inrow) ? cr * (uint32_t)a.Pp + (col ^ lds_swz(cr)) : 0u));
-                if (live && !inrow) {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const uint32_t le = l + (uint32_t)e;
-                        const uint32_t ce = fdiv(le, a.dRS);  // planes shorter than a slot pitch can be crossed twice
-                        const uint32_t pe = le - ce * RS;
-                        vset(qv[u], e, lds[ce * (uint32_t)a.Pp + ((pe + ((ce * RS) & 3u)) ^ lds_swz(ce))]);
-                    }
-                }
-                off[u] = live ? l * 4u : BUF_OOB;
-            }
-#pragma unroll
-            for (int u = 0; u < 4; ++u) buf_store<BUF_NT>(yr, off[u], qv[u]);
-        }
-    } else {
+    {
         // One wave per row, four rows in flight: everything about the row (its range [A, B) of whole lines,
         // where it ends, its swizzle) is wave-uniform and stays on the scalar unit; a lane only adds 4*k.
         const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
@@ -1416,8 +1388,10 @@ static bool make_line_args(const Geom& g, int numActive, const float* y, LineArg
     if (tune.ps > 0) a.psplit = tune.ps;
     a.P = (RS + a.psplit - 1) / a.psplit;
     a.psplit = (RS + a.P - 1) / a.P;
-    a.ext = a.psplit > 1 ? LINE_EXT : 0;
-    if (a.psplit > 1 && RS - (a.psplit - 1) * a.P < LINE_FLOATS) return false;  // last split must hold the extension
+    // A tile that takes whole planes writes one contiguous piece of y in k_gather_planar already.
+    if (a.psplit == 1) return false;
+    a.ext = LINE_EXT;
+    if (RS - (a.psplit - 1) * a.P < LINE_FLOATS) return false;  // the last split must hold the extension
     const int win = a.P + a.ext;
     ld = (win * lpp + threads - 1) / threads;
     if (ld < 4) ld = 4;
@@ -1430,7 +1404,6 @@ static bool make_line_args(const Geom& g, int numActive, const float* y, LineArg
     const bool aligned = (reinterpret_cast<uintptr_t>(y) & 127) == 0 && ((int64_t)a.Ct * RS) % LINE_FLOATS == 0 &&
                          ((int64_t)g.C * RS) % LINE_FLOATS == 0;
     a.spr = aligned ? (uint32_t)((a.P + LINE_EXT) / LINE_FLOATS * (LINE_FLOATS / 4)) : (uint32_t)((a.P + LINE_EXT + 3) / 4);
-    if (a.psplit == 1) a.spr = 1;  // unused: such a tile enumerates the chunk's slots directly
     a.tpb = (uint32_t)(a.psplit * a.cchunks);
     const uint64_t total = (uint64_t)numActive * a.tpb;
     if (total >= (1ull << 31)) return false;
@@ -1439,8 +1412,6 @@ static bool make_line_args(const Geom& g, int numActive, const float* y, LineArg
     a.dTpb = make_fastdiv(a.tpb);
     a.dPs = make_fastdiv((uint32_t)a.psplit);
     a.dS = make_fastdiv((uint32_t)g.S);
-    a.dSpr = make_fastdiv(a.spr);
-    a.dRS = make_fastdiv((uint32_t)RS);
     grid = a.total;
     return true;
 }
