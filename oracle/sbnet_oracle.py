@@ -166,3 +166,37 @@ def sparse_scatter_raw(x, M, idx, y, bsize, bstride, boffset, add, transpose, om
        int(bsize[0]), int(bsize[1]), int(bstride[0]), int(bstride[1]), int(M),
        idx.ctypes.data_as(_i16p), int(bool(add)), int(bool(transpose)), 0)
     return y
+
+
+# ---------------------------------------------------------------------------------------------
+# Gradients of the two differentiable ops, as the reference registers them
+# (sbnet_tensorflow/benchmark/sparse_conv_lib.py:80-147, sbnet_ops/tests/test_sparse_blocks.py:36-98):
+# compositions of the forward ops above, nothing else.
+# ---------------------------------------------------------------------------------------------
+
+def sparse_gather_grad(grad, x_shape, bin_counts, active_block_indices, dynamic_bsize, dynamic_bstride,
+                       dynamic_boffset, transpose=False):
+    """d(SparseGather)/dx (sparse_conv_lib.py:80-107): the block-shaped gradient scattered with
+    add=True, atomic=True onto zeros of x's shape, same transpose as the forward op."""
+    zeros = np.zeros(x_shape, dtype=np.float32)
+    return sparse_scatter(grad, bin_counts, active_block_indices, zeros, dynamic_bsize, dynamic_bstride,
+                          dynamic_boffset, add=True, atomic=True, transpose=transpose)
+
+
+def sparse_scatter_grad(grad, blocks_shape, bin_counts, active_block_indices, dynamic_bsize, dynamic_bstride,
+                        dynamic_boffset, add, transpose=False):
+    """(d/dblocks, d/dybase) of SparseScatter (sparse_conv_lib.py:110-147).
+
+    d/dblocks = sparse_gather(grad).  The reference calls the gather without the op's transpose attribute,
+    which yields an [M,R,S,C]-shaped gradient for an [M,C,R,S] input; here the gather takes the forward op's
+    transpose so the gradient has the input's layout (identical to the reference for transpose=False).
+    d/dybase = grad for add=True; for add=False grad times the stamp-out mask obtained by scattering blocks
+    of zeros over ones."""
+    d_blocks = sparse_gather(grad, bin_counts, active_block_indices, dynamic_bsize, dynamic_bstride,
+                             dynamic_boffset, transpose=transpose)
+    if add:
+        return d_blocks, grad.copy()
+    stamp = sparse_scatter(np.zeros(blocks_shape, dtype=np.float32), bin_counts, active_block_indices,
+                           np.ones_like(grad), dynamic_bsize, dynamic_bstride, dynamic_boffset, add=False,
+                           transpose=transpose)
+    return d_blocks, grad * stamp

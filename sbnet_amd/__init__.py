@@ -1,7 +1,8 @@
 """sbnet_amd: MI355X (gfx950) implementation of Sparse Blocks Network's three custom ops.
 
 `reduce_mask`, `sparse_gather`, `sparse_scatter` and `sparse_scatter_var` keep the reference's op
-names and arguments; they call hand-written HIP kernels through the C ABI of libsbnet_amd.so
+names and arguments (the gather and the copying scatter are differentiable, with the reference's
+gradient definitions); they call hand-written HIP kernels through the C ABI of libsbnet_amd.so
 (include/sbnet_amd.h).  Importing the package does not load the library; the first op call does,
 and raises if it has not been built.
 """
@@ -9,9 +10,10 @@ from .block_params import (BlockParams, calc_block_params, calc_block_params_res
                            calc_block_count_covering)
 from .ops import (HipError, InvalidArgument, ReduceMaskResult, reduce_mask, sparse_gather,  # noqa: F401
                   sparse_scatter, sparse_scatter_var)
+from .autograd import SparseGatherFunction, SparseScatterFunction  # noqa: F401
 
 __all__ = [
     "reduce_mask", "sparse_gather", "sparse_scatter", "sparse_scatter_var", "ReduceMaskResult",
-    "InvalidArgument", "HipError", "BlockParams", "calc_block_params", "calc_block_params_res_block",
+    "InvalidArgument", "HipError", "SparseGatherFunction", "SparseScatterFunction", "BlockParams", "calc_block_params", "calc_block_params_res_block",
     "calc_block_count_covering",
 ]

@@ -123,7 +123,21 @@ def reduce_mask(mask, dynamic_bcount, dynamic_bsize, dynamic_bstride, dynamic_bo
 def sparse_gather(x, bin_counts, active_block_indices, dynamic_bsize, dynamic_bstride, dynamic_boffset,
                   transpose=False, out=None):
     """SparseGather (sparse_gather.cc:48-57, 160-218): x [N,H,W,C] -> [M,bsize[0],bsize[1],C], or
-    [M,C,bsize[0],bsize[1]] with transpose=True, M = bin_counts[0]; out-of-image pixels read as 0."""
+    [M,C,bsize[0],bsize[1]] with transpose=True, M = bin_counts[0]; out-of-image pixels read as 0.
+    Differentiable with respect to x (sparse_conv_lib.py:80-107)."""
+    if torch.is_grad_enabled() and isinstance(x, torch.Tensor) and x.requires_grad:
+        if out is not None:
+            raise ValueError("out= cannot be combined with a differentiable input")
+        from .autograd import SparseGatherFunction
+        return SparseGatherFunction.apply(x, bin_counts, active_block_indices, dynamic_bsize, dynamic_bstride,
+                                          dynamic_boffset, bool(transpose))
+    return gather_forward(x, bin_counts, active_block_indices, dynamic_bsize, dynamic_bstride, dynamic_boffset,
+                          transpose, out)
+
+
+def gather_forward(x, bin_counts, active_block_indices, dynamic_bsize, dynamic_bstride, dynamic_boffset,
+                   transpose=False, out=None):
+    """The gather without autograd bookkeeping (what SparseGatherFunction.forward and the gradients call)."""
     lib = _lib.load()
     x = _dev_f32(x, "x")
     idx = _idx_i16(active_block_indices)
@@ -143,8 +157,9 @@ def sparse_gather(x, bin_counts, active_block_indices, dynamic_bsize, dynamic_bs
     return y
 
 
-def _scatter(x, bin_counts, active_block_indices, ybase, dynamic_bsize, dynamic_bstride, dynamic_boffset, add,
-             atomic, transpose, use_var):
+def scatter_forward(x, bin_counts, active_block_indices, ybase, dynamic_bsize, dynamic_bstride, dynamic_boffset, add,
+                    atomic, transpose, use_var):
+    """The scatter without autograd bookkeeping."""
     lib = _lib.load()
     x = _dev_f32(x, "x")
     idx = _idx_i16(active_block_indices)
@@ -181,13 +196,25 @@ def _scatter(x, bin_counts, active_block_indices, ybase, dynamic_bsize, dynamic_
 def sparse_scatter(x, bin_counts, active_block_indices, ybase, dynamic_bsize, dynamic_bstride, dynamic_boffset,
                    add, atomic=False, transpose=False):
     """SparseScatter (sparse_gather.cc:256-268, 286-357): returns copy(ybase) with the blocks of x written
-    (add=False), added (add=True) or atomically added (add=True, atomic=True) on top."""
-    return _scatter(x, bin_counts, active_block_indices, ybase, dynamic_bsize, dynamic_bstride, dynamic_boffset,
-                    add, atomic, transpose, use_var=False)
+    (add=False), added (add=True) or atomically added (add=True, atomic=True) on top.
+    Differentiable with respect to x and ybase (sparse_conv_lib.py:110-147)."""
+    if torch.is_grad_enabled() and ((isinstance(x, torch.Tensor) and x.requires_grad) or
+                                    (isinstance(ybase, torch.Tensor) and ybase.requires_grad)):
+        from .autograd import SparseScatterFunction
+        return SparseScatterFunction.apply(x, bin_counts, active_block_indices, ybase, dynamic_bsize,
+                                           dynamic_bstride, dynamic_boffset, bool(add), bool(atomic),
+                                           bool(transpose))
+    return scatter_forward(x, bin_counts, active_block_indices, ybase, dynamic_bsize, dynamic_bstride,
+                           dynamic_boffset, add, atomic, transpose, use_var=False)
 
 
 def sparse_scatter_var(x, bin_counts, active_block_indices, ybase, dynamic_bsize, dynamic_bstride,
                        dynamic_boffset, add, atomic=False, transpose=False):
-    """SparseScatterVar (sparse_gather.cc:242-254, 335-337): the same, in place on ybase, which is returned."""
-    return _scatter(x, bin_counts, active_block_indices, ybase, dynamic_bsize, dynamic_bstride, dynamic_boffset,
-                    add, atomic, transpose, use_var=True)
+    """SparseScatterVar (sparse_gather.cc:242-254, 335-337): the same, in place on ybase, which is returned.
+    The reference registers no gradient for this op (its ybase is a variable reference); neither does this."""
+    if torch.is_grad_enabled() and ((isinstance(x, torch.Tensor) and x.requires_grad) or
+                                    (isinstance(ybase, torch.Tensor) and ybase.requires_grad)):
+        raise NotImplementedError("sparse_scatter_var has no gradient (none is registered for SparseScatterVar "
+                                  "in the reference); use sparse_scatter, or call it under torch.no_grad()")
+    return scatter_forward(x, bin_counts, active_block_indices, ybase, dynamic_bsize, dynamic_bstride,
+                           dynamic_boffset, add, atomic, transpose, use_var=True)
