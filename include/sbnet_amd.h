@@ -172,11 +172,14 @@ size_t sbnet_sparse_scatter_workspace_bytes(int32_t num_active, const int64_t* y
  *   add=0 with overlapping blocks: as in the reference's GPU path, which block wins on an
  *   overlapped pixel is unspecified unless the overlapping values are equal.
  *   workspace   optional device scratch (4-byte aligned) of sbnet_sparse_scatter_workspace_bytes() bytes,
- *               or NULL.  It only matters for add=1, atomic=1, transpose=0: with it the overlapping adds
- *               are summed without atomics, each pixel by one owner, in ascending block-list order, so the
- *               result is bit-identical to the reference's sequential CPU functor and several times faster
- *               than hardware atomics.  Without it (or when more than 2x2 blocks cover a pixel, or the
- *               list names a block twice) hardware fp32 atomics are used: same sums up to fp32
+ *               or NULL.  It only matters for add=1, atomic=1; with it the overlapping adds need no atomics:
+ *               - transpose=0 and at most 2x2 blocks per pixel: each pixel is summed by one owner in ascending
+ *                 block-list order, bit-identical to the reference's sequential CPU functor;
+ *               - otherwise (transpose=1, or up to 16 blocks per pixel): ceil(R/U)*ceil(S/V) passes of plain
+ *                 adds, one class of mutually non-overlapping blocks per pass; reproducible, equal to the
+ *                 sequential sums up to fp32 reassociation.
+ *               Both run at streaming speed, several times faster than hardware atomics.  Without scratch, or
+ *               when the list names a block twice, hardware fp32 atomics are used: same sums up to fp32
  *               reassociation, in no particular order.
  */
 int sbnet_sparse_scatter(const float* x, int32_t num_active, const int16_t* active_block_indices,

@@ -117,9 +117,16 @@ int scatter_impl(const float* x, int32_t numActive, const int16_t* idx, float* o
     const sbnet::Geom g = make_geom((int)dims[0], (int)dims[1], (int)dims[2], (int)dims[3], bsize, bstride, boffset);
     const sbnet::ScatterMode mode =
         !add ? sbnet::SCATTER_ASSIGN : (atomic ? sbnet::SCATTER_ATOMIC : sbnet::SCATTER_ADD);
-    if (mode == sbnet::SCATTER_ATOMIC && !transpose && workspace) {
+    if (mode == sbnet::SCATTER_ATOMIC && workspace) {
+        // with scratch an "atomic" add needs no atomics: the owner-computes kernel where it applies (NHWC stack,
+        // at most 2x2 blocks per pixel; exact sequential order), else passes of plain adds over non-overlapping
+        // classes of blocks
         bool done = false;
-        SBNET_HIP(sbnet::launch_scatter_pull(x, out, idx, numActive, g, workspace, workspaceBytes, stream, done));
+        if (!transpose)
+            SBNET_HIP(sbnet::launch_scatter_pull(x, out, idx, numActive, g, workspace, workspaceBytes, stream, done));
+        if (done) return SBNET_OK;
+        SBNET_HIP(sbnet::launch_scatter_colored(x, out, idx, numActive, g, transpose != 0, workspace, workspaceBytes,
+                                                stream, done));
         if (done) return SBNET_OK;
     }
     SBNET_HIP(sbnet::launch_scatter(x, out, idx, numActive, g, transpose != 0, mode, stream));
@@ -229,7 +236,9 @@ size_t sbnet_sparse_scatter_workspace_bytes(int32_t num_active, const int64_t* y
         return 0;
     const sbnet::Geom g = make_geom((int)ybase_dims[0], (int)ybase_dims[1], (int)ybase_dims[2], (int)ybase_dims[3],
                                     bsize, bstride, boffset);
-    return sbnet::scatter_pull_workspace_bytes(g, num_active);
+    const size_t pull = sbnet::scatter_pull_workspace_bytes(g, num_active);
+    const size_t color = sbnet::scatter_color_workspace_bytes(g, num_active);
+    return pull > color ? pull : color;
 }
 
 int sbnet_sparse_scatter(const float* x, int32_t num_active, const int16_t* active_block_indices,

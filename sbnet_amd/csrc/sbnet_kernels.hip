@@ -104,6 +104,7 @@ __device__ __forceinline__ void commit(typename Vec<VEC>::type* dst, const typen
 // Reads the (n, bh, bw) triple of block ib (wave-uniform) and derives the block origin.
 struct BlockOrigin {
     int n, h0, w0;
+    int bh, bw;  // the block's grid position
     bool valid;  // n inside [0, N): guards against garbage rows in the index list
 };
 
@@ -112,8 +113,10 @@ __device__ __forceinline__ BlockOrigin load_origin(const int16_t* __restrict__ i
     BlockOrigin o;
     const int16_t* t = idx + (size_t)ib * 3;
     o.n = t[0];
-    o.h0 = g.oh + (int)t[1] * g.U;
-    o.w0 = g.ow + (int)t[2] * g.V;
+    o.bh = t[1];
+    o.bw = t[2];
+    o.h0 = g.oh + o.bh * g.U;
+    o.w0 = g.ow + o.bw * g.V;
     o.valid = (unsigned)o.n < (unsigned)g.N;
     return o;
 }
@@ -150,10 +153,37 @@ __device__ __forceinline__ BlockOrigin origin_of(const RawTriple& r, const Geom&
     const uint64_t bits = (((uint64_t)r.hi << 32) | r.lo) >> r.shift;
     BlockOrigin o;
     o.n = (int)(int16_t)(bits & 0xffffu);
-    o.h0 = g.oh + (int)(int16_t)((bits >> 16) & 0xffffu) * g.U;
-    o.w0 = g.ow + (int)(int16_t)((bits >> 32) & 0xffffu) * g.V;
+    o.bh = (int)(int16_t)((bits >> 16) & 0xffffu);
+    o.bw = (int)(int16_t)((bits >> 32) & 0xffffu);
+    o.h0 = g.oh + o.bh * g.U;
+    o.w0 = g.ow + o.bw * g.V;
     o.valid = (unsigned)o.n < (unsigned)g.N;
     return o;
+}
+
+// Overlapping scatter-add in passes ("colours").  Blocks whose grid positions agree modulo
+// (Kh, Kw) = (ceil(R/U), ceil(S/V)) cannot overlap, so a launch that handles one residue class can add
+// with plain load-add-store; Kh*Kw launches in a row cover the list.  The result is reproducible (the
+// order of the adds is the order of the passes) and runs at streaming speed, where hardware atomics reach
+// about a tenth of it.  A block listed twice breaks the premise: the map kernel of the pull scatter
+// detects that (`dup`), and then pass 0 handles every block with atomics and the other passes do nothing.
+constexpr int SCATTER_COLOR = 3;  // kernel-side mode; callers ask for SCATTER_ATOMIC
+
+struct ColorArgs {
+    int kh, kw, pass;
+    const int32_t* dup;
+};
+
+// True when this launch has nothing to do for the block; `atomics` tells how to add otherwise.
+__device__ __forceinline__ bool color_skip(const ColorArgs& col, const BlockOrigin& o, bool& atomics)
+{
+    typedef const int32_t __attribute__((address_space(4))) * const_i32_ptr;
+    atomics = *(const_i32_ptr)(reinterpret_cast<uintptr_t>(col.dup)) != 0;  // written by an earlier kernel
+    if (atomics) return col.pass != 0;
+    int mh = o.bh % col.kh, mw = o.bw % col.kw;
+    if (mh < 0) mh += col.kh;
+    if (mw < 0) mw += col.kw;
+    return mh * col.kw + mw != col.pass;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -222,7 +252,7 @@ __global__ __launch_bounds__(256) void k_gather_nhwc(const float* __restrict__ x
 // sparse_gather.cc:103-130 with transpose == false.
 template <int VEC, int MODE>
 __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ x, float* __restrict__ y,
-                                                      const int16_t* __restrict__ idx, NhwcArgs a)
+                                                      const int16_t* __restrict__ idx, NhwcArgs a, ColorArgs col)
 {
     typedef typename Vec<VEC>::type vec;
     const uint32_t lane = threadIdx.x & 63;
@@ -233,6 +263,8 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
     const uint32_t chunk = unit - ib * a.cpb;
     const BlockOrigin o = origin_of(load_triple(idx, ib), a.g);  // ib is wave-uniform: scalar load
     if (!o.valid) return;
+    bool atomics = MODE == SCATTER_ATOMIC;
+    if (MODE == SCATTER_COLOR && color_skip(col, o, atomics)) return;
     const int CV = a.g.C / VEC;
     const int slo = max(0, -o.w0), shi = min(a.g.S, a.g.W - o.w0);
     const int lo = slo * CV, hi = shi * CV;
@@ -257,7 +289,7 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
             }
         }
     }
-    if (MODE == SCATTER_ADD) {
+    if (MODE == SCATTER_ADD || (MODE == SCATTER_COLOR && !atomics)) {
         vec cur[NHWC_UNR];
 #pragma unroll
         for (int u = 0; u < NHWC_UNR; ++u)
@@ -265,10 +297,14 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
 #pragma unroll
         for (int u = 0; u < NHWC_UNR; ++u)
             if (dst[u] >= 0) st_stream(yv + dst[u], vadd(cur[u], v[u]));
+    } else if (MODE == SCATTER_ASSIGN) {
+#pragma unroll
+        for (int u = 0; u < NHWC_UNR; ++u)
+            if (dst[u] >= 0) commit<VEC, SCATTER_ASSIGN>(yv + dst[u], v[u]);
     } else {
 #pragma unroll
         for (int u = 0; u < NHWC_UNR; ++u)
-            if (dst[u] >= 0) commit<VEC, MODE>(yv + dst[u], v[u]);
+            if (dst[u] >= 0) commit<VEC, SCATTER_ATOMIC>(yv + dst[u], v[u]);
     }
 }
 
@@ -687,7 +723,7 @@ __global__ __launch_bounds__(512) void k_gather_lines(const float* __restrict__ 
 // sparse_gather.cc:103-130 with transpose == true: the block stack is [blocks, C, R, S].
 template <int VEC, int MODE>
 __global__ __launch_bounds__(512) void k_scatter_planar(const float* __restrict__ x, float* __restrict__ y,
-                                                        const int16_t* __restrict__ idx, TileArgs a)
+                                                        const int16_t* __restrict__ idx, TileArgs a, ColorArgs col)
 {
     typedef typename Vec<VEC>::type vec;
     extern __shared__ __attribute__((aligned(16))) float lds[];
@@ -696,6 +732,8 @@ __global__ __launch_bounds__(512) void k_scatter_planar(const float* __restrict_
     TileId t;
     decode_tile(a, blockIdx.x, t);
     const RawTriple raw = load_triple(idx, t.ib);  // scalar load, needed only after the barrier
+    bool atomics = MODE == SCATTER_ATOMIC;
+    if (MODE == SCATTER_COLOR && color_skip(col, origin_of(raw, a.g), atomics)) return;  // (here: before the loads)
 
     // global -> registers, planar side.  The last slot of a run, when partial, is read as the last 4 floats
     // of the run instead (overlapping its neighbour): no load leaves the run, no value needs fixing up.
@@ -752,7 +790,7 @@ __global__ __launch_bounds__(512) void k_scatter_planar(const float* __restrict_
     if (MODE == SCATTER_ASSIGN) {
 #pragma unroll
         for (int u = 0; u < TILE_LD; ++u) buf_store<BUF_NT>(yr, offs[u], w[u]);
-    } else if (MODE == SCATTER_ADD) {
+    } else if (MODE == SCATTER_ADD || (MODE == SCATTER_COLOR && !atomics)) {
         vec cur[TILE_LD];
 #pragma unroll
         for (int u = 0; u < TILE_LD; ++u) cur[u] = buf_load<VEC>(yr, offs[u]);
@@ -1477,7 +1515,8 @@ static void scatter_dispatch(const float* x, float* y, const int16_t* idx, const
     if (!transpose) {
         NhwcArgs a;
         if (!make_nhwc_args(g, numActive, VEC, a)) { err = hipErrorInvalidValue; return; }
-        hipLaunchKernelGGL((k_scatter_nhwc<VEC, MODE>), dim3((a.units + 3) / 4), dim3(256), 0, stream, x, y, idx, a);
+        hipLaunchKernelGGL((k_scatter_nhwc<VEC, MODE>), dim3((a.units + 3) / 4), dim3(256), 0, stream, x, y, idx, a,
+                           ColorArgs{1, 1, 0, nullptr});
     } else {
         TileArgs a;
         int threads;
@@ -1491,7 +1530,8 @@ static void scatter_dispatch(const float* x, float* y, const int16_t* idx, const
                                0, stream, x, y, idx, g, total);
             return;
         }
-        hipLaunchKernelGGL((k_scatter_planar<VEC, MODE>), dim3(grid), dim3(threads), lds, stream, x, y, idx, a);
+        hipLaunchKernelGGL((k_scatter_planar<VEC, MODE>), dim3(grid), dim3(threads), lds, stream, x, y, idx, a,
+                           ColorArgs{1, 1, 0, nullptr});
     }
 }
 
@@ -1517,16 +1557,11 @@ hipError_t launch_scatter(const float* x, float* y, const int16_t* idx, int numA
     return hipGetLastError();
 }
 
-// Geometry of the inverse block map of the pull scatter; false when the method does not apply.
-static bool make_pull_args(const Geom& g, int numActive, int vec, PullArgs& a, int64_t& mapN)
+// Extent of the inverse block map (blocks that can touch the image); false when it cannot be built.
+static bool make_map_args(const Geom& g, PullArgs& a, int64_t& mapN)
 {
     a.g = g;
-    const int Kh = (g.R + g.U - 1) / g.U, Kw = (g.S + g.V - 1) / g.V;
-    if ((2 * Kh - 1) * (2 * Kw - 1) > PULL_NB_MAX) return false;
-    a.kh1 = Kh - 1;
-    a.kw1 = Kw - 1;
-    a.tableStride = 1 + 2 * (2 * Kh - 1) * (2 * Kw - 1);
-    // blocks that can touch the image: oh + bh*U + R - 1 >= 0 and oh + bh*U <= H - 1 (floor divisions)
+    // oh + bh*U + R - 1 >= 0 and oh + bh*U <= H - 1 (floor divisions)
     auto floordiv = [](int64_t p, int64_t q) { return p >= 0 ? p / q : -((-p + q - 1) / q); };
     int64_t bhMin = -floordiv((int64_t)g.R - 1 + g.oh, g.U), bhMax = floordiv((int64_t)g.H - 1 - g.oh, g.U);
     int64_t bwMin = -floordiv((int64_t)g.S - 1 + g.ow, g.V), bwMax = floordiv((int64_t)g.W - 1 - g.ow, g.V);
@@ -1538,7 +1573,18 @@ static bool make_pull_args(const Geom& g, int numActive, int vec, PullArgs& a, i
     a.bhMin = (int)bhMin; a.bwMin = (int)bwMin;
     a.nBH = (int)(bhMax - bhMin + 1); a.nBW = (int)(bwMax - bwMin + 1);
     mapN = (int64_t)g.N * a.nBH * a.nBW;
-    if (mapN >= (1ll << 31)) return false;
+    return mapN < (1ll << 31);
+}
+
+// Geometry of the pull scatter; false when the method does not apply.
+static bool make_pull_args(const Geom& g, int numActive, int vec, PullArgs& a, int64_t& mapN)
+{
+    const int Kh = (g.R + g.U - 1) / g.U, Kw = (g.S + g.V - 1) / g.V;
+    if ((2 * Kh - 1) * (2 * Kw - 1) > PULL_NB_MAX) return false;
+    if (!make_map_args(g, a, mapN)) return false;
+    a.kh1 = Kh - 1;
+    a.kw1 = Kw - 1;
+    a.tableStride = 1 + 2 * (2 * Kh - 1) * (2 * Kw - 1);
     const uint64_t rowV = (uint64_t)g.S * g.C / vec, blockV = rowV * g.R;
     if (blockV >= (1ull << 31)) return false;
     a.CV = (uint32_t)(g.C / vec);
@@ -1587,6 +1633,87 @@ hipError_t launch_scatter_pull(const float* x, float* y, const int16_t* idx, int
     if (vec == 4) hipLaunchKernelGGL(k_scatter_pull<4>, dim3(wgs), dim3(256), 0, stream, x, y, idx, a, table, dup);
     else if (vec == 2) hipLaunchKernelGGL(k_scatter_pull<2>, dim3(wgs), dim3(256), 0, stream, x, y, idx, a, table, dup);
     else hipLaunchKernelGGL(k_scatter_pull<1>, dim3(wgs), dim3(256), 0, stream, x, y, idx, a, table, dup);
+    done = true;
+    return hipGetLastError();
+}
+
+// ---- scatter-add in passes ------------------------------------------------------------------
+
+constexpr int COLOR_MAX_PASSES = 16;
+
+size_t scatter_color_workspace_bytes(const Geom& g, int numActive)
+{
+    PullArgs a;
+    int64_t mapN = 0;
+    const int64_t Kh = ((int64_t)g.R + g.U - 1) / g.U, Kw = ((int64_t)g.S + g.V - 1) / g.V;
+    if (numActive <= 0 || Kh * Kw > COLOR_MAX_PASSES || !make_map_args(g, a, mapN)) return 0;
+    return (size_t)mapN * 4 + 16;
+}
+
+template <int VEC>
+static bool color_passes(const float* x, float* y, const int16_t* idx, const Geom& g, int numActive, bool transpose,
+                         ColorArgs col, int passes, hipStream_t stream)
+{
+    if (!transpose) {
+        NhwcArgs a;
+        if (!make_nhwc_args(g, numActive, VEC, a)) return false;
+        for (col.pass = 0; col.pass < passes; ++col.pass)
+            hipLaunchKernelGGL((k_scatter_nhwc<VEC, SCATTER_COLOR>), dim3((a.units + 3) / 4), dim3(256), 0, stream, x, y,
+                               idx, a, col);
+    } else {
+        TileArgs a;
+        int threads;
+        size_t lds;
+        unsigned grid;
+        if ((int64_t)g.R * g.S < 4 || !make_tile_args(g, numActive, VEC, a, threads, lds, grid, 16 * 1024)) return false;
+        for (col.pass = 0; col.pass < passes; ++col.pass)
+            hipLaunchKernelGGL((k_scatter_planar<VEC, SCATTER_COLOR>), dim3(grid), dim3(threads), lds, stream, x, y, idx,
+                               a, col);
+    }
+    return true;
+}
+
+hipError_t launch_scatter_colored(const float* x, float* y, const int16_t* idx, int numActive, const Geom& g,
+                                  bool transpose, void* workspace, size_t workspaceBytes, hipStream_t stream,
+                                  bool& done)
+{
+    done = false;
+    if (numActive == 0) { done = true; return hipSuccess; }
+    const size_t need = scatter_color_workspace_bytes(g, numActive);
+    if (!workspace || need == 0 || workspaceBytes < need || (reinterpret_cast<uintptr_t>(workspace) & 3))
+        return hipSuccess;
+    PullArgs pa;
+    int64_t mapN = 0;
+    if (!make_map_args(g, pa, mapN)) return hipSuccess;
+    ColorArgs col;
+    col.kh = (g.R + g.U - 1) / g.U;
+    col.kw = (g.S + g.V - 1) / g.V;
+    col.pass = 0;
+    int32_t* map = static_cast<int32_t*>(workspace);
+    int32_t* dup = map + mapN;
+    col.dup = dup;
+    // geometry checks first: nothing is launched unless the passes can run
+    const int vec = pick_vec(g, y, transpose ? nullptr : x);
+    {
+        NhwcArgs na;
+        TileArgs ta;
+        int threads;
+        size_t lds;
+        unsigned grid;
+        if (!transpose ? !make_nhwc_args(g, numActive, vec, na)
+                       : ((int64_t)g.R * g.S < 4 || !make_tile_args(g, numActive, vec, ta, threads, lds, grid, 16 * 1024)))
+            return hipSuccess;
+    }
+    int64_t fillWgs = (mapN + 255) / 256;
+    if (fillWgs > 4096) fillWgs = 4096;
+    if (fillWgs < 1) fillWgs = 1;
+    hipLaunchKernelGGL(k_pull_fill, dim3((unsigned)fillWgs), dim3(256), 0, stream, map, mapN, dup);
+    hipLaunchKernelGGL(k_pull_map, dim3((unsigned)((numActive + 255) / 256)), dim3(256), 0, stream, idx, numActive, pa,
+                       map, dup);
+    const int passes = col.kh * col.kw;
+    if (vec == 4) color_passes<4>(x, y, idx, g, numActive, transpose, col, passes, stream);
+    else if (vec == 2) color_passes<2>(x, y, idx, g, numActive, transpose, col, passes, stream);
+    else color_passes<1>(x, y, idx, g, numActive, transpose, col, passes, stream);
     done = true;
     return hipGetLastError();
 }

@@ -40,6 +40,14 @@ size_t scatter_pull_workspace_bytes(const Geom& g, int numActive);
 hipError_t launch_scatter_pull(const float* x, float* y, const int16_t* idx, int numActive, const Geom& g,
                                void* workspace, size_t workspaceBytes, hipStream_t stream, bool& done);
 
+// Scatter-add on overlapping blocks in ceil(R/U)*ceil(S/V) passes of plain load-add-store, one residue class of
+// block positions per pass (either stack layout, up to 16 passes): reproducible, within rounding of the
+// sequential order.  Needs scratch of scatter_color_workspace_bytes(); `done` as above.
+size_t scatter_color_workspace_bytes(const Geom& g, int numActive);
+hipError_t launch_scatter_colored(const float* x, float* y, const int16_t* idx, int numActive, const Geom& g,
+                                  bool transpose, void* workspace, size_t workspaceBytes, hipStream_t stream,
+                                  bool& done);
+
 hipError_t launch_copy(float* dst, const float* src, size_t count, hipStream_t stream);
 
 }  // namespace sbnet
