@@ -56,8 +56,11 @@ def test_scatter_workspace_query():
     # 16x16 blocks at stride 8: 2x2 blocks cover a pixel, the atomic-free method applies
     n = lib.sbnet_sparse_scatter_workspace_bytes(2000, dims, 4, I32x2(16, 16), 2, I32x2(8, 8), 2, I32x2(0, 0), 2)
     assert n >= 2 * 64 * 64 * 4 + 2000 * 4
-    # 16x16 at stride 4: 4x4 blocks cover a pixel, it does not
-    assert lib.sbnet_sparse_scatter_workspace_bytes(2000, dims, 4, I32x2(16, 16), 2, I32x2(4, 4), 2, I32x2(0, 0),
+    # 16x16 at stride 4: 4x4 blocks cover a pixel: the add runs in 16 passes, which needs the block map only
+    n = lib.sbnet_sparse_scatter_workspace_bytes(2000, dims, 4, I32x2(16, 16), 2, I32x2(4, 4), 2, I32x2(0, 0), 2)
+    assert 2 * 128 * 128 * 4 <= n < 2 * 140 * 140 * 4
+    # 16x16 at stride 3: 6x6 blocks cover a pixel, beyond both methods
+    assert lib.sbnet_sparse_scatter_workspace_bytes(2000, dims, 4, I32x2(16, 16), 2, I32x2(3, 3), 2, I32x2(0, 0),
                                                     2) == 0
     assert lib.sbnet_sparse_scatter_workspace_bytes(2000, dims, 3, I32x2(16, 16), 2, I32x2(8, 8), 2, I32x2(0, 0),
                                                     2) == 0
