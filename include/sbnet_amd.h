@@ -213,6 +213,16 @@ int sbnet_sparse_scatter_functor(const float* x, int N, int H, int W, int C, flo
    sparse_gather.cu:268-276) without its stream synchronisation.  count is in floats. */
 int sbnet_copy_tensor(float* dst, const float* src, size_t count, void* stream);
 
+/* Device timers: replace the CudaTimerStart / CudaTimerEnd ops (sparse_gather.cc:390-469) that the
+ * reference's benchmarks bracket their timed regions with.
+ *   sbnet_timer_start  creates an event, records it on `stream` and returns it as an opaque 64-bit handle
+ *                      (the reference passes the event to the end op the same way, as an int64 tensor).
+ *   sbnet_timer_end    records a second event on `stream`, waits for it, writes the elapsed device time in
+ *                      milliseconds to *dt_ms and destroys both events; a handle is good for one call.
+ * The reference records on the legacy default stream; pass NULL for that. */
+int sbnet_timer_start(void* stream, int64_t* start_event);
+int sbnet_timer_end(int64_t start_event, void* stream, float* dt_ms);
+
 #ifdef __cplusplus
 }
 #endif

@@ -48,6 +48,8 @@ SIGNATURES = {
     "sbnet_sparse_scatter_functor": (_int, [_vp, _int, _int, _int, _int, _vp] + [_int] * 7 + [_vp, _int, _int,
                                                                                               _int, _vp]),
     "sbnet_copy_tensor": (_int, [_vp, _vp, _sz, _vp]),
+    "sbnet_timer_start": (_int, [_vp, ctypes.POINTER(ctypes.c_int64)]),
+    "sbnet_timer_end": (_int, [ctypes.c_int64, _vp, ctypes.POINTER(ctypes.c_float)]),
 }
 
 _lib = None

@@ -301,4 +301,33 @@ int sbnet_copy_tensor(float* dst, const float* src, size_t count, void* stream)
     return SBNET_OK;
 }
 
+int sbnet_timer_start(void* stream, int64_t* start_event)
+{
+    if (!start_event) return SBNET_EINVAL_ARG;
+    hipEvent_t ev;
+    SBNET_HIP(hipEventCreate(&ev));
+    hipError_t e = hipEventRecord(ev, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) {
+        hipEventDestroy(ev);
+        return hip_fail(e);
+    }
+    *start_event = (int64_t)reinterpret_cast<intptr_t>(ev);
+    return SBNET_OK;
+}
+
+int sbnet_timer_end(int64_t start_event, void* stream, float* dt_ms)
+{
+    if (!start_event || !dt_ms) return SBNET_EINVAL_ARG;
+    hipEvent_t start = reinterpret_cast<hipEvent_t>((intptr_t)start_event);
+    hipEvent_t end;
+    SBNET_HIP(hipEventCreate(&end));
+    hipError_t e = hipEventRecord(end, static_cast<hipStream_t>(stream));
+    if (e == hipSuccess) e = hipEventSynchronize(end);
+    if (e == hipSuccess) e = hipEventElapsedTime(dt_ms, start, end);
+    hipEventDestroy(end);
+    hipEventDestroy(start);
+    if (e != hipSuccess) return hip_fail(e);
+    return SBNET_OK;
+}
+
 }  // extern "C"
