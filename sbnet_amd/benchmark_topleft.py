@@ -1,0 +1,161 @@
+"""Dense-versus-sparse benchmark on a synthetic top-left square mask.
+
+The reference's sweep (sbnet_tensorflow/benchmark/benchmark_topleft.py:63-133 with
+sparse_conv_perf.py:47-63, 163-262 and benchmark_configs.py): for each ResNet stage size, time the dense
+layer once, then for each target sparsity find the block size with the best sparse time and write one CSV row
+`H, W, C, K, BH, BW, sparsity, block_sparsity, dense_time, sparse_time, speedup` (times in milliseconds of
+device time, measured with the timer entry points of the op library around N_REPEAT back-to-back layers).
+
+Usage:
+    python -m sbnet_amd.benchmark_topleft --test [conv | res] --arch [resnet-50 | resnet-v2 | resnet-v3]
+                                          [--quick] [--out FILE]
+"""
+import argparse
+import collections
+import csv
+import math
+import sys
+import time
+
+import numpy as np
+import torch
+
+from . import sparse_conv as sc
+from .block_params import BlockParamError, calc_block_params, calc_block_params_res_block
+
+# benchmark_configs.py: [H, W, C, K] per ResNet stage
+INPUT_SIZE_DICT = {
+    "resnet-50": [[400, 700, 256, 64], [200, 350, 512, 128], [100, 175, 1024, 256], [50, 88, 2048, 512]],
+    "resnet-v2": [[400, 700, 96, 24], [200, 350, 192, 48], [100, 175, 256, 64], [50, 88, 384, 96]],
+    "resnet-v3": [[400, 700, 128, 32], [200, 350, 256, 64], [100, 175, 384, 96], [50, 88, 512, 128]],
+}
+SPARSITY_LIST = [0.6, 0.65, 0.7, 0.75, 0.8, 0.85, 0.9, 0.95, 0.99]
+BLOCK_SIZE_LIST_LIST = [range(11, 33, 2), range(7, 25, 2), range(5, 21, 2), range(5, 21, 2)]
+
+BATCH_SIZE = 1
+TOL = 0.05
+AVGPOOL = True
+N_REPEAT = 5
+N_WARMUP = 3
+N_RUN = 3
+
+PERF_RESULT_FIELDS = ["H", "W", "C", "K", "BH", "BW", "sparsity", "block_sparsity", "dense_time", "sparse_time",
+                      "speedup"]
+TestConfig = collections.namedtuple("TestConfig",
+                                    ["xsize", "ksize", "bsize", "strides", "padding", "is_sparse", "tol", "avgpool"])
+TestResult = collections.namedtuple("TestResult", ["avg_time", "block_sparsity"])
+
+
+def generate_top_left_mask(xsize, sparsity):
+    """sparse_conv_perf.py:47-63: a square of ones in the top-left corner with the target density."""
+    edge_ratio = math.sqrt(1.0 - sparsity)
+    height = int(math.ceil(edge_ratio * xsize[1]))
+    width = int(math.ceil(edge_ratio * xsize[2]))
+    x = np.zeros(xsize[:-1], dtype=np.float32)
+    x[:, :height, :width] = 1.0
+    return x
+
+
+def run_one(mask, config, res_block=False, device="cuda:0", n_warmup=N_WARMUP, n_run=N_RUN, n_repeat=N_REPEAT):
+    """sparse_conv_perf.py:208-262: average device milliseconds of one layer.  Inputs are created before the
+    timed region (one per repeat, as the reference does to defeat graph folding); the active-block list is
+    computed once before timing and reused, as the reference feeds it through placeholders."""
+    rng = np.random.RandomState(0)
+    x_init = torch.from_numpy(rng.uniform(-1, 1, config.xsize).astype(np.float32)).to(device)
+    C, K = config.ksize[2], config.ksize[3]
+    block_density = 1.0
+    with torch.no_grad():
+        if res_block:
+            ksize_list = [[1, 1, C, K], [3, 3, K, K], [1, 1, K, C]]
+            params = sc.BottleneckParams(ksize_list, device, seed=0)
+        else:
+            w = torch.from_numpy(rng.uniform(-1, 1, config.ksize).astype(np.float32)).to(device)
+        if config.is_sparse:
+            if res_block:
+                bp = calc_block_params_res_block(config.xsize, config.bsize, ksize_list, config.strides,
+                                                 config.padding)
+            else:
+                bp = calc_block_params(config.xsize, config.bsize, config.ksize, config.strides, config.padding)
+            ind = sc.convert_mask_to_indices_custom(torch.from_numpy(mask).to(device), bp, config.tol,
+                                                    config.avgpool)
+            block_density = int(ind.bin_counts[0]) / float(ind.active_block_indices.shape[0])
+            xs = [x_init.clone() for _ in range(n_repeat)]
+
+            def layer(i):
+                if res_block:
+                    return sc.sparse_res_block_bottleneck(xs[i], params, ind, bp, config.strides, True,
+                                                          data_format="NCHW", use_var=True)
+                return sc.sparse_conv2d_custom(xs[i], w, ind, bp, config.strides, use_var=True, transpose=True)
+        else:
+            xs = [x_init.permute(0, 3, 1, 2).contiguous() for _ in range(n_repeat)]   # NCHW, as the reference
+            w_oihw = None if res_block else w.permute(3, 2, 0, 1).contiguous()
+
+            def layer(i):
+                if res_block:
+                    return sc.res_block_bottleneck(xs[i], params, config.strides, True, data_format="NCHW")
+                return sc._conv_same_or_valid(xs[i], w_oihw, (config.strides[1], config.strides[2]), config.padding)
+
+        all_dt = []
+        for trial in range(n_warmup + n_run):
+            t0 = sc.hip_timer_start_op()
+            for i in range(n_repeat):
+                layer(i)
+            dt = sc.hip_timer_end_op(t0)
+            if trial >= n_warmup:
+                all_dt.append(dt)
+    return TestResult(avg_time=float(np.mean(all_dt)) / n_repeat, block_sparsity=1.0 - block_density)
+
+
+def sweep(test, arch, sparsities, block_size_lists, out, log=sys.stderr):
+    res_block = test == "res"
+    writer = csv.writer(out)
+    writer.writerow(PERF_RESULT_FIELDS)
+    for xsize, bsize_list in zip(INPUT_SIZE_DICT[arch], block_size_lists):
+        if test == "conv":
+            xsize_ = [BATCH_SIZE, xsize[0], xsize[1], xsize[3]]
+            ksize_ = [3, 3, xsize[3], xsize[3]]
+        else:
+            xsize_ = [BATCH_SIZE] + xsize[:-1]
+            ksize_ = [3, 3, xsize[2], xsize[3]]
+        dense_cfg = TestConfig(xsize_, ksize_, None, [1, 1, 1, 1], "SAME", False, None, None)
+        dense_time = run_one(None, dense_cfg, res_block=res_block).avg_time
+        for sparsity in sparsities:
+            best = None
+            mask = generate_top_left_mask(xsize_, sparsity)
+            for bsize in bsize_list:
+                if bsize > xsize[0] or bsize > xsize[1]:
+                    continue
+                cfg = TestConfig(xsize_, ksize_, [1, bsize, bsize, 1], [1, 1, 1, 1], "SAME", True, TOL, AVGPOOL)
+                try:
+                    r = run_one(mask, cfg, res_block=res_block)
+                except BlockParamError:
+                    continue  # the reference's geometry asserts reject this block size for this input
+                if best is None or r.avg_time < best[1].avg_time:
+                    best = (bsize, r)
+            if best is None:
+                continue
+            row = [xsize[0], xsize[1], xsize[2], xsize[3], best[0], best[0], sparsity,
+                   round(best[1].block_sparsity, 4), round(dense_time, 4), round(best[1].avg_time, 4),
+                   round(dense_time / best[1].avg_time, 3)]
+            writer.writerow(row)
+            out.flush()
+            print("%s %s %s" % (test, arch, dict(zip(PERF_RESULT_FIELDS, row))), file=log, flush=True)
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description="Sparse convolution / residual block benchmark, top-left mask")
+    ap.add_argument("--test", default="conv", choices=["conv", "res"])
+    ap.add_argument("--arch", default="resnet-v2", choices=sorted(INPUT_SIZE_DICT))
+    ap.add_argument("--quick", action="store_true", help="three sparsities, three block sizes per stage")
+    ap.add_argument("--out", default=None, help="CSV file (default: ours_topleft_<test>_<timestamp>.csv)")
+    args = ap.parse_args(argv)
+    sparsities = [0.6, 0.9, 0.99] if args.quick else SPARSITY_LIST
+    blists = [list(b)[::4] for b in BLOCK_SIZE_LIST_LIST] if args.quick else BLOCK_SIZE_LIST_LIST
+    name = args.out or "ours_topleft_%s_%s.csv" % (args.test, time.strftime("%Y%m%d_%H%M%S"))
+    print("Writing output to %s" % name, file=sys.stderr)
+    with open(name, "w", newline="") as f:
+        sweep(args.test, args.arch, sparsities, blists, f)
+
+
+if __name__ == "__main__":
+    main()

@@ -162,3 +162,25 @@ def test_timer_twins_measure_device_time():
     ref = ref0.elapsed_time(ref1)
     assert isinstance(dt, float) and dt > 0.0
     assert 0.5 * ref < dt < 2.0 * ref + 0.5
+
+
+def test_benchmark_run_one_dense_and_sparse():
+    """run_one of the top-left-mask benchmark (sparse_conv_perf.py:208-262) on a small stage: times are positive
+    and the block sparsity follows from the mask: a top-left square of density 0.25 on 40x60 with 5x5 input
+    blocks (3x3 outputs) activates ceil-covered blocks only."""
+    from sbnet_amd import benchmark_topleft as bt
+    xsize, ksize = [1, 40, 60, 16], [3, 3, 16, 4]
+    dense = bt.run_one(None, bt.TestConfig(xsize, ksize, None, [1, 1, 1, 1], "SAME", False, None, None),
+                       res_block=True, n_warmup=1, n_run=1, n_repeat=2)
+    assert dense.avg_time > 0 and dense.block_sparsity == 0.0
+    mask = bt.generate_top_left_mask(xsize, 0.75)
+    assert mask.shape == (1, 40, 60) and mask.sum() == 20 * 30 and mask[0, :20, :30].all()
+    for res_block in (False, True):
+        k = ksize if res_block else [3, 3, 16, 16]
+        r = bt.run_one(mask, bt.TestConfig(xsize, k, [1, 5, 5, 1], [1, 1, 1, 1], "SAME", True, bt.TOL, bt.AVGPOOL),
+                       res_block=res_block, n_warmup=1, n_run=1, n_repeat=2)
+        assert r.avg_time > 0
+        # blocks start at -1 + 3*b and are active when more than 5 % of 25 pixels are set: rows b <= 6 (start 17,
+        # 3 rows inside), columns b <= 10 (start 29: 1 column inside, 5/25 > 0.05): 7 x 11 of the 13 x 20 blocks that
+        # calc_block_params lays over 40 x 60
+        assert abs(r.block_sparsity - (1.0 - 7 * 11 / (13 * 20.0))) < 1e-6
