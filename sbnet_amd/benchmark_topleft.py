@@ -8,7 +8,7 @@ device time, measured with the timer entry points of the op library around N_REP
 
 Usage:
     python -m sbnet_amd.benchmark_topleft --test [conv | res] --arch [resnet-50 | resnet-v2 | resnet-v3]
-                                          [--quick] [--out FILE]
+                                          [--quick] [--graph] [--out FILE]
 """
 import argparse
 import collections
@@ -56,10 +56,15 @@ def generate_top_left_mask(xsize, sparsity):
     return x
 
 
-def run_one(mask, config, res_block=False, device="cuda:0", n_warmup=N_WARMUP, n_run=N_RUN, n_repeat=N_REPEAT):
+def run_one(mask, config, res_block=False, device="cuda:0", n_warmup=N_WARMUP, n_run=N_RUN, n_repeat=N_REPEAT,
+            use_graph=False):
     """sparse_conv_perf.py:208-262: average device milliseconds of one layer.  Inputs are created before the
     timed region (one per repeat, as the reference does to defeat graph folding); the active-block list is
-    computed once before timing and reused, as the reference feeds it through placeholders."""
+    computed once before timing and reused, as the reference feeds it through placeholders.
+
+    use_graph captures the n_repeat layers into one HIP graph and times replays: the reference runs inside a
+    TensorFlow graph with no per-op Python cost, and at high sparsity an eagerly launched sparse layer is
+    bound by host launch time (about 15 launches per residual block), not by the device."""
     rng = np.random.RandomState(0)
     x_init = torch.from_numpy(rng.uniform(-1, 1, config.xsize).astype(np.float32)).to(device)
     C, K = config.ksize[2], config.ksize[3]
@@ -95,18 +100,34 @@ def run_one(mask, config, res_block=False, device="cuda:0", n_warmup=N_WARMUP, n
                     return sc.res_block_bottleneck(xs[i], params, config.strides, True, data_format="NCHW")
                 return sc._conv_same_or_valid(xs[i], w_oihw, (config.strides[1], config.strides[2]), config.padding)
 
+        def repeats():
+            for i in range(n_repeat):
+                layer(i)
+
+        run = repeats
+        if use_graph:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                repeats()   # library handles, workspaces and algorithm choices are settled outside the capture
+                repeats()
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                repeats()
+            run = graph.replay
         all_dt = []
         for trial in range(n_warmup + n_run):
             t0 = sc.hip_timer_start_op()
-            for i in range(n_repeat):
-                layer(i)
+            run()
             dt = sc.hip_timer_end_op(t0)
             if trial >= n_warmup:
                 all_dt.append(dt)
     return TestResult(avg_time=float(np.mean(all_dt)) / n_repeat, block_sparsity=1.0 - block_density)
 
 
-def sweep(test, arch, sparsities, block_size_lists, out, log=sys.stderr):
+def sweep(test, arch, sparsities, block_size_lists, out, log=sys.stderr, use_graph=False):
     res_block = test == "res"
     writer = csv.writer(out)
     writer.writerow(PERF_RESULT_FIELDS)
@@ -118,7 +139,7 @@ def sweep(test, arch, sparsities, block_size_lists, out, log=sys.stderr):
             xsize_ = [BATCH_SIZE] + xsize[:-1]
             ksize_ = [3, 3, xsize[2], xsize[3]]
         dense_cfg = TestConfig(xsize_, ksize_, None, [1, 1, 1, 1], "SAME", False, None, None)
-        dense_time = run_one(None, dense_cfg, res_block=res_block).avg_time
+        dense_time = run_one(None, dense_cfg, res_block=res_block, use_graph=use_graph).avg_time
         for sparsity in sparsities:
             best = None
             mask = generate_top_left_mask(xsize_, sparsity)
@@ -127,7 +148,7 @@ def sweep(test, arch, sparsities, block_size_lists, out, log=sys.stderr):
                     continue
                 cfg = TestConfig(xsize_, ksize_, [1, bsize, bsize, 1], [1, 1, 1, 1], "SAME", True, TOL, AVGPOOL)
                 try:
-                    r = run_one(mask, cfg, res_block=res_block)
+                    r = run_one(mask, cfg, res_block=res_block, use_graph=use_graph)
                 except BlockParamError:
                     continue  # the reference's geometry asserts reject this block size for this input
                 if best is None or r.avg_time < best[1].avg_time:
@@ -147,6 +168,7 @@ def main(argv=None):
     ap.add_argument("--test", default="conv", choices=["conv", "res"])
     ap.add_argument("--arch", default="resnet-v2", choices=sorted(INPUT_SIZE_DICT))
     ap.add_argument("--quick", action="store_true", help="three sparsities, three block sizes per stage")
+    ap.add_argument("--graph", action="store_true", help="time HIP-graph replays instead of eager launches")
     ap.add_argument("--out", default=None, help="CSV file (default: ours_topleft_<test>_<timestamp>.csv)")
     args = ap.parse_args(argv)
     sparsities = [0.6, 0.9, 0.99] if args.quick else SPARSITY_LIST
@@ -154,7 +176,7 @@ def main(argv=None):
     name = args.out or "ours_topleft_%s_%s.csv" % (args.test, time.strftime("%Y%m%d_%H%M%S"))
     print("Writing output to %s" % name, file=sys.stderr)
     with open(name, "w", newline="") as f:
-        sweep(args.test, args.arch, sparsities, blists, f)
+        sweep(args.test, args.arch, sparsities, blists, f, use_graph=args.graph)
 
 
 if __name__ == "__main__":

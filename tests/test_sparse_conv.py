@@ -184,3 +184,47 @@ def test_benchmark_run_one_dense_and_sparse():
         # 3 rows inside), columns b <= 10 (start 29: 1 column inside, 5/25 > 0.05): 7 x 11 of the 13 x 20 blocks that
         # calc_block_params lays over 40 x 60
         assert abs(r.block_sparsity - (1.0 - 7 * 11 / (13 * 20.0))) < 1e-6
+
+
+@pytest.mark.parametrize("data_format", ["NHWC", "NCHW"])
+def test_sparse_res_block_in_a_hip_graph_replays_identically(data_format):
+    """The three block ops enqueue on the caller's stream and allocate nothing of their own, so a whole sparse
+    residual block can be captured into a HIP graph.  Every replay, with eager work and synchronisation in
+    between, must reproduce the eager result for the input present at replay time."""
+    import sbnet_amd
+    from sbnet_amd import sparse_conv as sc
+    rnd = np.random.RandomState(2)
+    ch = 16
+    shape = [2, 30, 40, ch]
+    mask = (rnd.uniform(0, 1, shape[:3]) > 0.8).astype(np.float32)
+    ksize_list = [[1, 1, ch, ch // 4], [3, 3, ch // 4, ch // 4], [1, 1, ch // 4, ch]]
+    bp = sbnet_amd.calc_block_params_res_block(shape, [1, 7, 7, 1], ksize_list, [1, 1, 1, 1], "SAME")
+    params = sc.BottleneckParams(ksize_list, DEV, seed=7)
+    ind = sc.convert_mask_to_indices_custom(torch.from_numpy(mask).to(DEV), bp, 0.0)
+    x_static = torch.zeros(shape, device=DEV)
+
+    def layer():
+        return sc.sparse_res_block_bottleneck(x_static, params, ind, bp, [1, 1, 1, 1], is_training=False,
+                                              data_format=data_format)
+
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            layer()
+            layer()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            y_static = layer()
+        for rep in range(4):
+            xval = torch.from_numpy(rnd.uniform(-1, 1, shape).astype(np.float32)).to(DEV)
+            x_static.copy_(xval)
+            graph.replay()
+            torch.cuda.synchronize()
+            got = y_static.clone()
+            exp = sc.sparse_res_block_bottleneck(xval, params, ind, bp, [1, 1, 1, 1], is_training=False,
+                                                 data_format=data_format)
+            torch.cuda.synchronize()
+            np.testing.assert_array_equal(got.cpu().numpy(), exp.cpu().numpy())
