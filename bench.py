@@ -173,6 +173,23 @@ class Path:
                                                      self.sbo, 2, int(wl.s_add), int(wl.s_atomic), int(wl.transpose),
                                                      s["out"].data_ptr(), wp, wn, self.stream))
 
+    def step_device_count(self, i):
+        """The same three ops with the count left on the device (entry points with the _device_count suffix):
+        launches are sized for the whole list (max_active = N*bcount_h*bcount_w) and nothing waits for the host."""
+        s, wl = self.sets[i], self.wl
+        if "stack_cap" not in s:
+            R, S = wl.bsize
+            s["stack_cap"] = self.torch.empty((self.maxidx, self.C, R, S) if wl.transpose else
+                                              (self.maxidx, R, S, self.C), dtype=self.torch.float32, device="cuda:0")
+        self.reduce(i, sync=False)
+        self.check(self.lib.sbnet_sparse_gather_device_count(
+            s["x"].data_ptr(), self.dims, 4, s["dcount"].data_ptr(), self.maxidx, s["idx"].data_ptr(), self.bs, 2,
+            self.bst, 2, self.bo, 2, int(wl.transpose), s["stack_cap"].data_ptr(), self.stream))
+        self.check(self.lib.sbnet_sparse_scatter_var_device_count(
+            s["stack_cap"].data_ptr(), s["dcount"].data_ptr(), self.maxidx, s["idx"].data_ptr(), s["base"].data_ptr(),
+            self.dims, 4, self.sbs, 2, self.sbst, 2, self.sbo, 2, int(wl.s_add), int(wl.s_atomic), int(wl.transpose),
+            None, 0, self.stream))
+
     def step(self, i):
         M = self.reduce(i) if self.wl.mask is not None else self.M
         if self.wl.x is not None:
@@ -325,6 +342,21 @@ def main():
     step_bytes = sum(path.bytes.values())
     value = step_bytes / (ms_per_step * 1e-3) * 1e-9
 
+    # the same pipeline without the host-visible count (not the reference's contract; reported beside `value`)
+    for i in range(max(args.warmup, nsets)):
+        path.step_device_count(i % nsets)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        path.step_device_count(i % nsets)
+    torch.cuda.synchronize()
+    dc_ms = (time.perf_counter() - t0) / args.steps * 1e3
+    dc_counts = [int(s["dcount"].cpu()[0]) for s in path.sets]
+    assert dc_counts == [path.M] * nsets, "device-resident count differs from the host-visible one"
+    for s in path.sets:
+        s.pop("stack_cap", None)
+    torch.cuda.empty_cache()
+
     ops = path.op_table()
     g = ops["gather"]
     roofline = {"bound": "hbm", "kernel": "k_gather_lines<5> (sparse_gather, transpose=True)",
@@ -342,6 +374,11 @@ def main():
                                % (round(args.density * 100), path.M),
                    "buffer_sets": nsets, "bytes_per_step": step_bytes},
         "ops": ops, "roofline": roofline,
+        "pipeline_device_count": {"ms_per_step": round(dc_ms, 4),
+                                  "GBps": round(step_bytes / (dc_ms * 1e-3) * 1e-9, 1),
+                                  "max_active": path.maxidx,
+                                  "note": "count read on the device, launches sized for max_active blocks, "
+                                          "no host sync inside a step"},
     }
     if not args.no_cpu:
         nb = path.bytes["gather"] + path.bytes["scatter"]

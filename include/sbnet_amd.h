@@ -213,6 +213,42 @@ int sbnet_sparse_scatter_functor(const float* x, int N, int H, int W, int C, flo
    sparse_gather.cu:268-276) without its stream synchronisation.  count is in floats. */
 int sbnet_copy_tensor(float* dst, const float* src, size_t count, void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Variants that take the block count from device memory
+ * ------------------------------------------------------------------------------------------
+ * These have no counterpart in the reference, whose gather and scatter read bin_counts from host memory
+ * (sparse_gather.cc:190-192, 315-317) and therefore force a device-to-host copy and a stream
+ * synchronisation after every reduce_mask.  They are for callers that must not wait on the host: a pipeline
+ * captured into a HIP graph, a serving loop that enqueues reduce_mask -> gather -> ... -> scatter without
+ * stalling.  bin_counts_device is the int32 that sbnet_reduce_mask leaves in bin_counts_device; max_active is
+ * the capacity of the list and of the block stack (N*bcount[0]*bcount[1] always suffices): the launch is sized
+ * for max_active blocks and workgroups of blocks at or beyond *bin_counts_device return at once.  Only the
+ * first *bin_counts_device blocks of y (gather) are written / of x (scatter) are read.  All other arguments,
+ * checks and results are those of the entry points without the suffix. */
+int sbnet_sparse_gather_device_count(const float* x, const int64_t* x_dims, int x_rank,
+                                     const int32_t* bin_counts_device, int32_t max_active,
+                                     const int16_t* active_block_indices,
+                                     const int32_t* bsize, int bsize_len,
+                                     const int32_t* bstride, int bstride_len,
+                                     const int32_t* boffset, int boffset_len,
+                                     int transpose, float* y, void* stream);
+int sbnet_sparse_scatter_device_count(const float* x, const int32_t* bin_counts_device, int32_t max_active,
+                                      const int16_t* active_block_indices,
+                                      const float* ybase, const int64_t* ybase_dims, int ybase_rank,
+                                      const int32_t* bsize, int bsize_len,
+                                      const int32_t* bstride, int bstride_len,
+                                      const int32_t* boffset, int boffset_len,
+                                      int add, int atomic, int transpose, float* y,
+                                      void* workspace, size_t workspace_bytes, void* stream);
+int sbnet_sparse_scatter_var_device_count(const float* x, const int32_t* bin_counts_device, int32_t max_active,
+                                          const int16_t* active_block_indices,
+                                          float* ybase, const int64_t* ybase_dims, int ybase_rank,
+                                          const int32_t* bsize, int bsize_len,
+                                          const int32_t* bstride, int bstride_len,
+                                          const int32_t* boffset, int boffset_len,
+                                          int add, int atomic, int transpose,
+                                          void* workspace, size_t workspace_bytes, void* stream);
+
 /* Device timers: replace the CudaTimerStart / CudaTimerEnd ops (sparse_gather.cc:390-469) that the
  * reference's benchmarks bracket their timed regions with.
  *   sbnet_timer_start  creates an event, records it on `stream` and returns it as an opaque 64-bit handle

@@ -47,6 +47,12 @@ SIGNATURES = {
                                         _int, _int, _int, _vp, _sz, _vp]),
     "sbnet_sparse_scatter_functor": (_int, [_vp, _int, _int, _int, _int, _vp] + [_int] * 7 + [_vp, _int, _int,
                                                                                               _int, _vp]),
+    "sbnet_sparse_gather_device_count": (_int, [_vp, _i64p, _int, _vp, _i32, _vp, _i32p, _int, _i32p, _int, _i32p,
+                                                _int, _int, _vp, _vp]),
+    "sbnet_sparse_scatter_device_count": (_int, [_vp, _vp, _i32, _vp, _vp, _i64p, _int, _i32p, _int, _i32p, _int,
+                                                 _i32p, _int, _int, _int, _int, _vp, _vp, _sz, _vp]),
+    "sbnet_sparse_scatter_var_device_count": (_int, [_vp, _vp, _i32, _vp, _vp, _i64p, _int, _i32p, _int, _i32p, _int,
+                                                     _i32p, _int, _int, _int, _int, _vp, _sz, _vp]),
     "sbnet_copy_tensor": (_int, [_vp, _vp, _sz, _vp]),
     "sbnet_timer_start": (_int, [_vp, ctypes.POINTER(ctypes.c_int64)]),
     "sbnet_timer_end": (_int, [ctypes.c_int64, _vp, ctypes.POINTER(ctypes.c_float)]),

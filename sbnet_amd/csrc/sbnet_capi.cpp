@@ -45,6 +45,7 @@ sbnet::Geom make_geom(int N, int H, int W, int C, const int32_t* bsize, const in
     g.R = bsize[0]; g.S = bsize[1];
     g.U = bstride[0]; g.V = bstride[1];
     g.oh = boffset[0]; g.ow = boffset[1];
+    g.countDev = nullptr;
     return g;
 }
 
@@ -104,7 +105,20 @@ int reduce_mask_impl(const float* mask, int N, int H, int W, const int32_t* bcou
     return SBNET_OK;
 }
 
-int scatter_impl(const float* x, int32_t numActive, const int16_t* idx, float* out,
+int gather_impl(const float* x, int N, int H, int W, int C, float* y, const int32_t* bsize, const int32_t* bstride,
+                const int32_t* boffset, int numActive, const int32_t* countDev, const int16_t* idx, int transpose,
+                hipStream_t stream)
+{
+    if (numActive < 0) return SBNET_EINVAL_ARG;
+    if (numActive > 0 && (!x || !y || !idx)) return SBNET_EINVAL_ARG;
+    if (!geom_ok(N, H, W, C, bsize, bstride)) return SBNET_EINVAL_ARG;
+    sbnet::Geom g = make_geom(N, H, W, C, bsize, bstride, boffset);
+    g.countDev = countDev;
+    SBNET_HIP(sbnet::launch_gather(x, y, idx, numActive, g, transpose != 0, stream));
+    return SBNET_OK;
+}
+
+int scatter_impl(const float* x, int32_t numActive, const int32_t* countDev, const int16_t* idx, float* out,
                  const int64_t* dims, const int32_t* bsize, const int32_t* bstride,
                  const int32_t* boffset, int add, int atomic, int transpose, void* workspace,
                  size_t workspaceBytes, hipStream_t stream)
@@ -114,7 +128,8 @@ int scatter_impl(const float* x, int32_t numActive, const int16_t* idx, float* o
     if (!out || !dims_fit_int(dims)) return SBNET_EINVAL_ARG;
     if (!geom_ok((int)dims[0], (int)dims[1], (int)dims[2], (int)dims[3], bsize, bstride))
         return SBNET_EINVAL_ARG;
-    const sbnet::Geom g = make_geom((int)dims[0], (int)dims[1], (int)dims[2], (int)dims[3], bsize, bstride, boffset);
+    sbnet::Geom g = make_geom((int)dims[0], (int)dims[1], (int)dims[2], (int)dims[3], bsize, bstride, boffset);
+    g.countDev = countDev;
     const sbnet::ScatterMode mode =
         !add ? sbnet::SCATTER_ASSIGN : (atomic ? sbnet::SCATTER_ATOMIC : sbnet::SCATTER_ADD);
     if (mode == sbnet::SCATTER_ATOMIC && workspace) {
@@ -217,13 +232,23 @@ int sbnet_sparse_gather_functor(const float* x, int N, int H, int W, int C, floa
                                 const int16_t* activeBlockIndices, int transpose, void* stream)
 {
     const int32_t bsize[2] = {bSzH, bSzW}, bstride[2] = {bStrH, bStrW}, boffset[2] = {bOffsH0, bOffsW0};
-    if (numActive < 0) return SBNET_EINVAL_ARG;
-    if (numActive > 0 && (!x || !y || !activeBlockIndices)) return SBNET_EINVAL_ARG;
-    if (!geom_ok(N, H, W, C, bsize, bstride)) return SBNET_EINVAL_ARG;
-    const sbnet::Geom g = make_geom(N, H, W, C, bsize, bstride, boffset);
-    SBNET_HIP(sbnet::launch_gather(x, y, activeBlockIndices, numActive, g, transpose != 0,
-                                   static_cast<hipStream_t>(stream)));
-    return SBNET_OK;
+    return gather_impl(x, N, H, W, C, y, bsize, bstride, boffset, numActive, nullptr, activeBlockIndices, transpose,
+                       static_cast<hipStream_t>(stream));
+}
+
+int sbnet_sparse_gather_device_count(const float* x, const int64_t* x_dims, int x_rank,
+                                     const int32_t* bin_counts_device, int32_t max_active,
+                                     const int16_t* active_block_indices, const int32_t* bsize, int bsize_len,
+                                     const int32_t* bstride, int bstride_len, const int32_t* boffset,
+                                     int boffset_len, int transpose, float* y, void* stream)
+{
+    if (x_rank != 4) return SBNET_EINVAL_RANK;
+    if (!pair_ok(bsize, bsize_len) || !pair_ok(bstride, bstride_len) || !pair_ok(boffset, boffset_len))
+        return SBNET_EINVAL_PARAM_SHAPE;
+    if (!x_dims || !dims_fit_int(x_dims) || !bin_counts_device) return SBNET_EINVAL_ARG;
+    return gather_impl(x, (int)x_dims[0], (int)x_dims[1], (int)x_dims[2], (int)x_dims[3], y, bsize, bstride, boffset,
+                       max_active, bin_counts_device, active_block_indices, transpose,
+                       static_cast<hipStream_t>(stream));
 }
 
 size_t sbnet_sparse_scatter_workspace_bytes(int32_t num_active, const int64_t* ybase_dims, int ybase_rank,
@@ -241,11 +266,11 @@ size_t sbnet_sparse_scatter_workspace_bytes(int32_t num_active, const int64_t* y
     return pull > color ? pull : color;
 }
 
-int sbnet_sparse_scatter(const float* x, int32_t num_active, const int16_t* active_block_indices,
-                         const float* ybase, const int64_t* ybase_dims, int ybase_rank,
-                         const int32_t* bsize, int bsize_len, const int32_t* bstride, int bstride_len,
-                         const int32_t* boffset, int boffset_len, int add, int atomic, int transpose,
-                         float* y, void* workspace, size_t workspace_bytes, void* stream)
+static int scatter_op(const float* x, int32_t num_active, const int32_t* bin_counts_device,
+                      const int16_t* active_block_indices, const float* ybase, const int64_t* ybase_dims,
+                      int ybase_rank, const int32_t* bsize, int bsize_len, const int32_t* bstride, int bstride_len,
+                      const int32_t* boffset, int boffset_len, int add, int atomic, int transpose, float* y,
+                      void* workspace, size_t workspace_bytes, void* stream)
 {
     // order of checks as in sparse_gather.cc:307-327
     if (!pair_ok(bsize, bsize_len) || !pair_ok(bstride, bstride_len) || !pair_ok(boffset, boffset_len))
@@ -263,8 +288,47 @@ int sbnet_sparse_scatter(const float* x, int32_t num_active, const int16_t* acti
     if (!geom_ok((int)ybase_dims[0], (int)ybase_dims[1], (int)ybase_dims[2], (int)ybase_dims[3], bsize, bstride))
         return SBNET_EINVAL_ARG;
     SBNET_HIP(sbnet::launch_copy(y, ybase, count, s));  // sparse_gather.cc:338-346, no stream sync
-    return scatter_impl(x, num_active, active_block_indices, y, ybase_dims, bsize, bstride, boffset, add,
-                        atomic, transpose, workspace, workspace_bytes, s);
+    return scatter_impl(x, num_active, bin_counts_device, active_block_indices, y, ybase_dims, bsize, bstride, boffset,
+                        add, atomic, transpose, workspace, workspace_bytes, s);
+}
+
+int sbnet_sparse_scatter(const float* x, int32_t num_active, const int16_t* active_block_indices,
+                         const float* ybase, const int64_t* ybase_dims, int ybase_rank,
+                         const int32_t* bsize, int bsize_len, const int32_t* bstride, int bstride_len,
+                         const int32_t* boffset, int boffset_len, int add, int atomic, int transpose,
+                         float* y, void* workspace, size_t workspace_bytes, void* stream)
+{
+    return scatter_op(x, num_active, nullptr, active_block_indices, ybase, ybase_dims, ybase_rank, bsize, bsize_len,
+                      bstride, bstride_len, boffset, boffset_len, add, atomic, transpose, y, workspace,
+                      workspace_bytes, stream);
+}
+
+int sbnet_sparse_scatter_device_count(const float* x, const int32_t* bin_counts_device, int32_t max_active,
+                                      const int16_t* active_block_indices, const float* ybase,
+                                      const int64_t* ybase_dims, int ybase_rank, const int32_t* bsize, int bsize_len,
+                                      const int32_t* bstride, int bstride_len, const int32_t* boffset,
+                                      int boffset_len, int add, int atomic, int transpose, float* y,
+                                      void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (!bin_counts_device) return SBNET_EINVAL_ARG;
+    return scatter_op(x, max_active, bin_counts_device, active_block_indices, ybase, ybase_dims, ybase_rank, bsize,
+                      bsize_len, bstride, bstride_len, boffset, boffset_len, add, atomic, transpose, y, workspace,
+                      workspace_bytes, stream);
+}
+
+static int scatter_var_op(const float* x, int32_t num_active, const int32_t* bin_counts_device,
+                          const int16_t* active_block_indices, float* ybase, const int64_t* ybase_dims,
+                          int ybase_rank, const int32_t* bsize, int bsize_len, const int32_t* bstride,
+                          int bstride_len, const int32_t* boffset, int boffset_len, int add, int atomic,
+                          int transpose, void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (!pair_ok(bsize, bsize_len) || !pair_ok(bstride, bstride_len) || !pair_ok(boffset, boffset_len))
+        return SBNET_EINVAL_PARAM_SHAPE;
+    if (!atomic && add && !(bstride[0] >= bsize[0] && bstride[1] >= bsize[1])) return SBNET_EINVAL_OVERLAP;
+    if (ybase_rank != 4) return SBNET_EINVAL_RANK;
+    if (!ybase || !ybase_dims) return SBNET_EINVAL_ARG;
+    return scatter_impl(x, num_active, bin_counts_device, active_block_indices, ybase, ybase_dims, bsize, bstride,
+                        boffset, add, atomic, transpose, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
 int sbnet_sparse_scatter_var(const float* x, int32_t num_active, const int16_t* active_block_indices,
@@ -274,13 +338,22 @@ int sbnet_sparse_scatter_var(const float* x, int32_t num_active, const int16_t* 
                              int atomic, int transpose, void* workspace, size_t workspace_bytes,
                              void* stream)
 {
-    if (!pair_ok(bsize, bsize_len) || !pair_ok(bstride, bstride_len) || !pair_ok(boffset, boffset_len))
-        return SBNET_EINVAL_PARAM_SHAPE;
-    if (!atomic && add && !(bstride[0] >= bsize[0] && bstride[1] >= bsize[1])) return SBNET_EINVAL_OVERLAP;
-    if (ybase_rank != 4) return SBNET_EINVAL_RANK;
-    if (!ybase || !ybase_dims) return SBNET_EINVAL_ARG;
-    return scatter_impl(x, num_active, active_block_indices, ybase, ybase_dims, bsize, bstride, boffset,
-                        add, atomic, transpose, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+    return scatter_var_op(x, num_active, nullptr, active_block_indices, ybase, ybase_dims, ybase_rank, bsize,
+                          bsize_len, bstride, bstride_len, boffset, boffset_len, add, atomic, transpose, workspace,
+                          workspace_bytes, stream);
+}
+
+int sbnet_sparse_scatter_var_device_count(const float* x, const int32_t* bin_counts_device, int32_t max_active,
+                                          const int16_t* active_block_indices, float* ybase,
+                                          const int64_t* ybase_dims, int ybase_rank, const int32_t* bsize,
+                                          int bsize_len, const int32_t* bstride, int bstride_len,
+                                          const int32_t* boffset, int boffset_len, int add, int atomic,
+                                          int transpose, void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (!bin_counts_device) return SBNET_EINVAL_ARG;
+    return scatter_var_op(x, max_active, bin_counts_device, active_block_indices, ybase, ybase_dims, ybase_rank,
+                          bsize, bsize_len, bstride, bstride_len, boffset, boffset_len, add, atomic, transpose,
+                          workspace, workspace_bytes, stream);
 }
 
 int sbnet_sparse_scatter_functor(const float* x, int N, int H, int W, int C, float* y, int bOffsH0,
@@ -290,7 +363,7 @@ int sbnet_sparse_scatter_functor(const float* x, int N, int H, int W, int C, flo
 {
     const int32_t bsize[2] = {bSzH, bSzW}, bstride[2] = {bStrH, bStrW}, boffset[2] = {bOffsH0, bOffsW0};
     const int64_t dims[4] = {N, H, W, C};
-    return scatter_impl(x, numActive, activeBlockIndices, y, dims, bsize, bstride, boffset, add, atomic,
+    return scatter_impl(x, numActive, nullptr, activeBlockIndices, y, dims, bsize, bstride, boffset, add, atomic,
                         transpose, nullptr, 0, static_cast<hipStream_t>(stream));
 }
 

@@ -161,6 +161,14 @@ __device__ __forceinline__ BlockOrigin origin_of(const RawTriple& r, const Geom&
     return o;
 }
 
+// True for list rows at or beyond the device-resident count (see Geom::countDev); ib is wave-uniform.
+__device__ __forceinline__ bool beyond_count(const Geom& g, uint32_t ib)
+{
+    if (!g.countDev) return false;
+    typedef const int32_t __attribute__((address_space(4))) * const_i32_ptr;
+    return ib >= (uint32_t)*(const_i32_ptr)(reinterpret_cast<uintptr_t>(g.countDev));
+}
+
 // Overlapping scatter-add in passes ("colours").  Blocks whose grid positions agree modulo
 // (Kh, Kw) = (ceil(R/U), ceil(S/V)) cannot overlap, so a launch that handles one residue class can add
 // with plain load-add-store; Kh*Kw launches in a row cover the list.  The result is reproducible (the
@@ -217,6 +225,7 @@ __global__ __launch_bounds__(256) void k_gather_nhwc(const float* __restrict__ x
     if (unit >= a.units) return;
     unit = __builtin_amdgcn_readfirstlane(unit);
     const uint32_t ib = fdiv(unit, a.dCpb);
+    if (beyond_count(a.g, ib)) return;
     const uint32_t chunk = unit - ib * a.cpb;
     const BlockOrigin o = origin_of(load_triple(idx, ib), a.g);  // ib is wave-uniform: scalar load
     const int CV = a.g.C / VEC;
@@ -260,6 +269,7 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
     if (unit >= a.units) return;
     unit = __builtin_amdgcn_readfirstlane(unit);
     const uint32_t ib = fdiv(unit, a.dCpb);
+    if (beyond_count(a.g, ib)) return;
     const uint32_t chunk = unit - ib * a.cpb;
     const BlockOrigin o = origin_of(load_triple(idx, ib), a.g);  // ib is wave-uniform: scalar load
     if (!o.valid) return;
@@ -474,6 +484,7 @@ __global__ __launch_bounds__(512) void k_gather_planar(const float* __restrict__
     const uint32_t RS = (uint32_t)(a.g.R * a.g.S);
     TileId t;
     decode_tile(a, blockIdx.x, t);
+    if (beyond_count(a.g, t.ib)) return;
     const BlockOrigin o = origin_of(load_triple(idx, t.ib), a.g);
     // a block index outside [0, N) gets an empty descriptor: every load returns 0
     const rsrc_t xr = make_rsrc(x + (o.valid ? (int64_t)o.n * a.imgFloats : 0), o.valid ? a.imgBytes : 0u);
@@ -593,6 +604,7 @@ __global__ __launch_bounds__(512) void k_gather_lines(const float* __restrict__ 
         }
     }
     const uint32_t ib = fdiv(id, a.dTpb);
+    if (beyond_count(a.g, ib)) return;
     const uint32_t rem = id - ib * a.tpb;
     const uint32_t cc = fdiv(rem, a.dPs);
     const uint32_t split = rem - cc * (uint32_t)a.psplit;
@@ -731,6 +743,7 @@ __global__ __launch_bounds__(512) void k_scatter_planar(const float* __restrict_
     const uint32_t RS = (uint32_t)(a.g.R * a.g.S);
     TileId t;
     decode_tile(a, blockIdx.x, t);
+    if (beyond_count(a.g, t.ib)) return;
     const RawTriple raw = load_triple(idx, t.ib);  // scalar load, needed only after the barrier
     bool atomics = MODE == SCATTER_ATOMIC;
     if (MODE == SCATTER_COLOR && color_skip(col, origin_of(raw, a.g), atomics)) return;  // (here: before the loads)
@@ -820,6 +833,7 @@ __global__ __launch_bounds__(256) void k_planar_small(const float* __restrict__ 
         const int c = (int)(i % g.C);
         const int p = (int)((i / g.C) % RS);
         const int64_t ib = i / ((int64_t)g.C * RS);
+        if (g.countDev && ib >= *g.countDev) continue;
         const int r = p / g.S, s = p - r * g.S;
         const BlockOrigin o = load_origin(idx, (uint32_t)ib, g);
         const int hh = o.h0 + r, ww = o.w0 + s;
@@ -1074,7 +1088,7 @@ __global__ __launch_bounds__(256) void k_pull_map(const int16_t* __restrict__ id
                                                   int32_t* __restrict__ map, int32_t* __restrict__ dup)
 {
     const int ib = (int)(blockIdx.x * 256 + threadIdx.x);
-    if (ib >= numActive) return;
+    if (ib >= numActive || (a.g.countDev && ib >= *a.g.countDev)) return;
     const int64_t slot = pull_slot(a, idx[(size_t)ib * 3], idx[(size_t)ib * 3 + 1], idx[(size_t)ib * 3 + 2]);
     if (slot < 0) return;  // this block cannot touch the image
     if (atomicCAS(map + slot, -1, ib) != -1) *dup = 1;
@@ -1084,7 +1098,7 @@ __global__ __launch_bounds__(256) void k_pull_table(const int16_t* __restrict__ 
                                                     const int32_t* __restrict__ map, int32_t* __restrict__ table)
 {
     const int ib = (int)(blockIdx.x * 256 + threadIdx.x);
-    if (ib >= numActive) return;
+    if (ib >= numActive || (a.g.countDev && ib >= *a.g.countDev)) return;
     const int n = idx[(size_t)ib * 3], bh = idx[(size_t)ib * 3 + 1], bw = idx[(size_t)ib * 3 + 2];
     int ids[PULL_NB_MAX], offs[PULL_NB_MAX];
     int cnt = 0;
@@ -1125,6 +1139,7 @@ __global__ __launch_bounds__(256) void k_scatter_pull(const float* __restrict__ 
     if (unit >= a.units) return;
     unit = __builtin_amdgcn_readfirstlane(unit);
     const uint32_t ib = fdiv(unit, a.dCpb);
+    if (beyond_count(a.g, ib)) return;
     const uint32_t chunk = unit - ib * a.cpb;
     const BlockOrigin o = origin_of(load_triple(idx, ib), a.g);  // ib is wave-uniform: scalar load
     if (!o.valid) return;

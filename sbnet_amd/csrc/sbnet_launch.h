@@ -15,6 +15,10 @@ struct Geom {
     int R, S;    // block size  (bsize)
     int U, V;    // block stride (bstride)
     int oh, ow;  // block offset (boffset)
+    // Optional: device-resident length of the block list.  When set, the kernels treat numActive as the
+    // capacity of the list and skip rows at or beyond *countDev, so no host round trip is needed between
+    // reduce_mask and its consumers.
+    const int32_t* countDev;
 };
 
 enum ScatterMode { SCATTER_ASSIGN = 0, SCATTER_ADD = 1, SCATTER_ATOMIC = 2 };

@@ -70,6 +70,16 @@ def _count(bin_counts):
     return int(np.asarray(bin_counts).reshape(-1)[0])
 
 
+def _device_count(bin_counts):
+    """A bin_counts that is still on the GPU (reduce_mask(..., sync=False)) selects the entry points that read
+    the count on the device; returns the int32 tensor, or None for a host-side count."""
+    if isinstance(bin_counts, torch.Tensor) and bin_counts.is_cuda:
+        if bin_counts.dtype != torch.int32 or bin_counts.numel() < 1:
+            raise TypeError("a device-resident bin_counts must be an int32 tensor with one element")
+        return bin_counts
+    return None
+
+
 def _stream():
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
@@ -141,7 +151,9 @@ def gather_forward(x, bin_counts, active_block_indices, dynamic_bsize, dynamic_b
     lib = _lib.load()
     x = _dev_f32(x, "x")
     idx = _idx_i16(active_block_indices)
-    M = _count(bin_counts)
+    dcount = _device_count(bin_counts)
+    # with a device-resident count the stack is sized for the whole list and only its first rows are written
+    M = int(idx.shape[0]) if dcount is not None else _count(bin_counts)
     bs, bsp, bsl = _pair(dynamic_bsize)
     bt, btp, btl = _pair(dynamic_bstride)
     bo, bop, bol = _pair(dynamic_boffset)
@@ -152,8 +164,14 @@ def gather_forward(x, bin_counts, active_block_indices, dynamic_bsize, dynamic_b
             C, R, S = int(x.shape[3]), int(bs[0]), int(bs[1])
             shape = (M, C, R, S) if transpose else (M, R, S, C)
             y = torch.empty(shape, dtype=torch.float32, device=x.device)
-        _check(lib.sbnet_sparse_gather(x.data_ptr(), dims, rank, M, idx.data_ptr(), bsp, bsl, btp, btl, bop, bol,
-                                       int(bool(transpose)), y.data_ptr() if y is not None else None, _stream()))
+        yp = y.data_ptr() if y is not None else None
+        if dcount is not None:
+            _check(lib.sbnet_sparse_gather_device_count(x.data_ptr(), dims, rank, dcount.data_ptr(), M, idx.data_ptr(),
+                                                        bsp, bsl, btp, btl, bop, bol, int(bool(transpose)), yp,
+                                                        _stream()))
+        else:
+            _check(lib.sbnet_sparse_gather(x.data_ptr(), dims, rank, M, idx.data_ptr(), bsp, bsl, btp, btl, bop, bol,
+                                           int(bool(transpose)), yp, _stream()))
     return y
 
 
@@ -163,7 +181,8 @@ def scatter_forward(x, bin_counts, active_block_indices, ybase, dynamic_bsize, d
     lib = _lib.load()
     x = _dev_f32(x, "x")
     idx = _idx_i16(active_block_indices)
-    M = _count(bin_counts)
+    dcount = _device_count(bin_counts)
+    M = min(int(idx.shape[0]), int(x.shape[0])) if dcount is not None else _count(bin_counts)
     if not isinstance(ybase, torch.Tensor) or not ybase.is_cuda or ybase.dtype != torch.float32:
         raise TypeError("ybase must be a float32 tensor on the GPU")
     if use_var and not ybase.is_contiguous():
@@ -181,15 +200,25 @@ def scatter_forward(x, bin_counts, active_block_indices, ybase, dynamic_bsize, d
             if need:
                 ws = _workspace(ybase.device, need)
                 ws_ptr, ws_bytes = ws.data_ptr(), ws.numel()
+        flags = (int(bool(add)), int(bool(atomic)), int(bool(transpose)))
         if use_var:
-            _check(lib.sbnet_sparse_scatter_var(x.data_ptr(), M, idx.data_ptr(), ybase.data_ptr(), dims, rank,
-                                                bsp, bsl, btp, btl, bop, bol, int(bool(add)), int(bool(atomic)),
-                                                int(bool(transpose)), ws_ptr, ws_bytes, _stream()))
+            if dcount is not None:
+                _check(lib.sbnet_sparse_scatter_var_device_count(x.data_ptr(), dcount.data_ptr(), M, idx.data_ptr(),
+                                                                 ybase.data_ptr(), dims, rank, bsp, bsl, btp, btl,
+                                                                 bop, bol, *flags, ws_ptr, ws_bytes, _stream()))
+            else:
+                _check(lib.sbnet_sparse_scatter_var(x.data_ptr(), M, idx.data_ptr(), ybase.data_ptr(), dims, rank,
+                                                    bsp, bsl, btp, btl, bop, bol, *flags, ws_ptr, ws_bytes,
+                                                    _stream()))
             return ybase
         y = torch.empty_like(ybase)
-        _check(lib.sbnet_sparse_scatter(x.data_ptr(), M, idx.data_ptr(), ybase.data_ptr(), dims, rank, bsp, bsl,
-                                        btp, btl, bop, bol, int(bool(add)), int(bool(atomic)),
-                                        int(bool(transpose)), y.data_ptr(), ws_ptr, ws_bytes, _stream()))
+        if dcount is not None:
+            _check(lib.sbnet_sparse_scatter_device_count(x.data_ptr(), dcount.data_ptr(), M, idx.data_ptr(),
+                                                         ybase.data_ptr(), dims, rank, bsp, bsl, btp, btl, bop, bol,
+                                                         *flags, y.data_ptr(), ws_ptr, ws_bytes, _stream()))
+        else:
+            _check(lib.sbnet_sparse_scatter(x.data_ptr(), M, idx.data_ptr(), ybase.data_ptr(), dims, rank, bsp, bsl,
+                                            btp, btl, bop, bol, *flags, y.data_ptr(), ws_ptr, ws_bytes, _stream()))
         return y
 
 

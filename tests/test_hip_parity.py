@@ -522,6 +522,105 @@ def test_overlapping_add_in_passes_with_repeated_blocks():
     np.testing.assert_array_equal(host(y), y_o)
 
 
+@pytest.mark.parametrize("geom", [
+    # (N, H, W, C), bsize, bstride, boffset
+    ((2, 40, 52, 8), (6, 6), (6, 6), (-2, -1)),            # tiling
+    ((2, 40, 52, 8), (6, 6), (3, 3), (-2, -1)),            # overlapping 2x2: owner-computes add / passes
+    ((1, 120, 130, 32), (27, 27), (25, 25), (-1, -1)),     # planes split over tiles (line-owning gather)
+    ((3, 20, 20, 4), (1, 3), (1, 3), (0, 0)),              # planes below 4 pixels (generic planar kernel)
+    ((1, 30, 30, 6), (7, 7), (2, 2), (0, 0)),              # 4x4 blocks per pixel, 2-channel vectors
+])
+def test_device_resident_count(geom):
+    """reduce_mask(sync=False) leaves the count on the GPU; gather and scatter given that tensor read it there,
+    are launched for the whole list capacity and must touch only the first `count` blocks."""
+    (N, H, W, C), bs, bst, bo = geom
+    rng = np.random.default_rng(C * 100 + H)
+    bc = bcount_covering(H, W, bst, bo)
+    # isolated mask pixels at a rate that leaves about half of the blocks active
+    mask = (rng.random((N, H, W, 1)) < 1.0 - 0.5 ** (1.0 / (bs[0] * bs[1]))).astype(np.float32)
+    x = rng.integers(-8, 9, size=(N, H, W, C)).astype(np.float32)
+    tol = 0.5
+    idx_o, cnt_o = orc.reduce_mask(mask, bc, bs, bst, bo, tol, False)
+    M, cap = int(cnt_o[0]), N * bc[0] * bc[1]
+    assert 0 < M < cap
+    r = sbnet_amd.reduce_mask(dev(mask), bc, bs, bst, bo, tol=tol, avgpool=False, sync=False)
+    assert r.bin_counts.is_cuda
+    overlap = bst[0] < bs[0] or bst[1] < bs[1]
+    xd = dev(x)
+    for transpose in (False, True):
+        g_o = orc.sparse_gather(x, cnt_o, idx_o, bs, bst, bo, transpose=transpose)
+        shape = (cap,) + g_o.shape[1:]
+        out = torch.full(shape, 555.0, dtype=torch.float32, device=DEV)
+        g = sbnet_amd.sparse_gather(xd, r.bin_counts, r.active_block_indices, bs, bst, bo, transpose=transpose,
+                                    out=out)
+        assert tuple(g.shape) == shape
+        np.testing.assert_array_equal(host(g[:M]), g_o)
+        assert float(g[M:].min()) == 555.0 and float(g[M:].max()) == 555.0
+        # rows of the stack past the count hold values that must not reach the tensor
+        g[M:] = 1.0e6
+        base = rng.integers(-4, 5, size=(N, H, W, C)).astype(np.float32)
+        for add, atomic in ((False, False), (True, True)) if overlap else ((False, False), (True, False), (True, True)):
+            if not add and overlap:
+                continue  # overlapping plain writes of different blocks race on the GPU
+            y_o = orc.sparse_scatter(g_o, cnt_o, idx_o, base, bs, bst, bo, add=add, atomic=atomic,
+                                     transpose=transpose)
+            y = sbnet_amd.sparse_scatter(g, r.bin_counts, r.active_block_indices, dev(base), bs, bst, bo, add=add,
+                                         atomic=atomic, transpose=transpose)
+            np.testing.assert_array_equal(host(y), y_o)
+            yv = dev(base)
+            sbnet_amd.sparse_scatter_var(g, r.bin_counts, r.active_block_indices, yv, bs, bst, bo, add=add,
+                                         atomic=atomic, transpose=transpose)
+            np.testing.assert_array_equal(host(yv), y_o)
+
+
+def test_whole_pipeline_in_a_hip_graph():
+    """reduce_mask -> gather -> scatter_var captured once and replayed on different masks and inputs: with the
+    count on the device nothing in the pipeline waits for the host, and every replay must match the oracle."""
+    rng = np.random.default_rng(99)
+    N, H, W, C = 1, 120, 130, 32
+    bs, bst, bo = (27, 27), (25, 25), (-1, -1)
+    bc = bcount_covering(H, W, bst, bo)
+    cap = N * bc[0] * bc[1]
+    mask_s = torch.zeros((N, H, W, 1), device=DEV)
+    x_s = torch.zeros((N, H, W, C), device=DEV)
+    y_s = torch.zeros((N, H, W, C), device=DEV)
+    stack_s = torch.zeros((cap, C, bs[0], bs[1]), device=DEV)
+
+    def pipeline():
+        r = sbnet_amd.reduce_mask(mask_s, bc, bs, bst, bo, tol=0.5, avgpool=False, sync=False)
+        sbnet_amd.sparse_gather(x_s, r.bin_counts, r.active_block_indices, bs, bst, bo, transpose=True, out=stack_s)
+        sbnet_amd.sparse_scatter_var(stack_s, r.bin_counts, r.active_block_indices, y_s, bs, bst, bo, add=False,
+                                     transpose=True)
+        return r
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        pipeline()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        r = pipeline()
+    for rep in range(4):
+        mask = (rng.random((N, H, W, 1)) < 0.0008 * (rep + 1)).astype(np.float32)
+        x = rng.standard_normal((N, H, W, C)).astype(np.float32)
+        mask_s.copy_(dev(mask))
+        x_s.copy_(dev(x))
+        y_s.fill_(-3.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        idx_o, cnt_o = orc.reduce_mask(mask, bc, bs, bst, bo, 0.5, False)
+        M = int(cnt_o[0])
+        assert int(r.bin_counts.cpu()[0]) == M
+        np.testing.assert_array_equal(host(r.active_block_indices)[:M], idx_o[:M])
+        g_o = orc.sparse_gather(x, cnt_o, idx_o, bs, bst, bo, transpose=True)
+        np.testing.assert_array_equal(host(stack_s[:M]), g_o)
+        y_o = orc.sparse_scatter(g_o, cnt_o, idx_o, np.full_like(x, -3.0), bs, bst, bo, add=False, transpose=True)
+        np.testing.assert_array_equal(host(y_s), y_o)
+
+
 # ---------------------------------------------------------------------------------------------
 # functor-level entry points and the copy
 # ---------------------------------------------------------------------------------------------
