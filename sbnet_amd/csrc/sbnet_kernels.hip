@@ -1380,7 +1380,8 @@ static bool make_tile_args(const Geom& g, int numActive, int vec, TileArgs& a, i
         threads = nthr;
         if (maxP >= RS) break;
     }
-    if (tune.wg > 0 && tune.wg != threads) return false;  // experiments must pick a consistent size
+    if (tune.wg > 0 && tune.wg < threads) return false;  // experiments must pick a sufficient size
+    if (tune.wg > 0) threads = tune.wg;
     if (maxP < 1) return false;
     a.psplit = (RS + maxP - 1) / maxP;
     a.P = (RS + a.psplit - 1) / a.psplit;

@@ -621,6 +621,56 @@ def test_whole_pipeline_in_a_hip_graph():
         np.testing.assert_array_equal(host(y_s), y_o)
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_random_geometries(seed):
+    """Seeded random block geometries (sizes, strides, offsets on either side of zero, channel counts of every
+    vector width, partial channel chunks, planes from 1 to ~1200 pixels), random block lists in random order
+    with off-image and out-of-range rows: every op and mode against the oracle."""
+    rng = np.random.default_rng(1000 + seed)
+    for case in range(6):
+        N = int(rng.integers(1, 4))
+        C = int(rng.choice([1, 2, 3, 4, 6, 8, 12, 20, 32, 36, 48, 64, 68]))
+        R, S = int(rng.integers(1, 36)), int(rng.integers(1, 36))
+        U = int(rng.integers(max(1, R // 2), R + 3))
+        V = int(rng.integers(max(1, S // 2), S + 3))
+        H, W = int(rng.integers(R, 3 * R + 20)), int(rng.integers(S, 3 * S + 20))
+        bo = (int(rng.integers(-R + 1, 3)), int(rng.integers(-S + 1, 3)))
+        bc = bcount_covering(H, W, (U, V), bo)
+        cells = [(n, i, j) for n in range(N) for i in range(bc[0]) for j in range(bc[1]) if rng.random() < 0.6]
+        cells += [(0, 0, 0), (N - 1, bc[0] - 1, bc[1] - 1)]
+        cells = sorted(set(cells))
+        idx = np.array(cells, np.int16)
+        rng.shuffle(idx, axis=0)
+        M = len(idx)
+        cnt = np.array([M], np.int32)
+        bs, bst = (R, S), (U, V)
+        tag = "seed %d case %d: N%d H%d W%d C%d bs %s bst %s bo %s M %d" % (seed, case, N, H, W, C, bs, bst, bo, M)
+        x = rng.integers(-8, 9, size=(N, H, W, C)).astype(np.float32)
+        base = rng.integers(-4, 5, size=(N, H, W, C)).astype(np.float32)
+        overlap = U < R or V < S
+        xd, idxd = dev(x), dev(idx)
+        for transpose in (False, True):
+            g_o = orc.sparse_gather(x, cnt, idx, bs, bst, bo, transpose=transpose)
+            g = sbnet_amd.sparse_gather(xd, cnt, idxd, bs, bst, bo, transpose=transpose)
+            np.testing.assert_array_equal(host(g), g_o, err_msg=tag)
+            stack = rng.integers(-8, 9, size=g_o.shape).astype(np.float32)
+            sd = dev(stack)
+            modes = [(True, True)] if overlap else [(False, False), (True, False), (True, True)]
+            for add, atomic in modes:
+                y_o = orc.sparse_scatter(stack, cnt, idx, base, bs, bst, bo, add=add, atomic=atomic,
+                                         transpose=transpose)
+                yv = dev(base)
+                sbnet_amd.sparse_scatter_var(sd, cnt, idxd, yv, bs, bst, bo, add=add, atomic=atomic,
+                                             transpose=transpose)
+                np.testing.assert_array_equal(host(yv), y_o, err_msg=tag + " add %s atomic %s T %s" %
+                                              (add, atomic, transpose))
+            if overlap:
+                # plain writes of identical values: order-free
+                y_o = orc.sparse_scatter(g_o, cnt, idx, base, bs, bst, bo, add=False, transpose=transpose)
+                y = sbnet_amd.sparse_scatter(g, cnt, idxd, dev(base), bs, bst, bo, add=False, transpose=transpose)
+                np.testing.assert_array_equal(host(y), y_o, err_msg=tag)
+
+
 # ---------------------------------------------------------------------------------------------
 # functor-level entry points and the copy
 # ---------------------------------------------------------------------------------------------
