@@ -216,7 +216,7 @@ struct NhwcArgs {
 
 // sparse_gather.cc:67-88 with transpose == false.
 template <int VEC>
-__global__ __launch_bounds__(256) void k_gather_nhwc(const float* __restrict__ x, float* __restrict__ y,
+__global__ __launch_bounds__(256) void k_gather_nhwc_wide(const float* __restrict__ x, float* __restrict__ y,
                                                      const int16_t* __restrict__ idx, NhwcArgs a)
 {
     typedef typename Vec<VEC>::type vec;
@@ -260,7 +260,7 @@ __global__ __launch_bounds__(256) void k_gather_nhwc(const float* __restrict__ x
 
 // sparse_gather.cc:103-130 with transpose == false.
 template <int VEC, int MODE>
-__global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ x, float* __restrict__ y,
+__global__ __launch_bounds__(256) void k_scatter_nhwc_wide(const float* __restrict__ x, float* __restrict__ y,
                                                       const int16_t* __restrict__ idx, NhwcArgs a, ColorArgs col)
 {
     typedef typename Vec<VEC>::type vec;
@@ -440,6 +440,112 @@ template <int AUX> __device__ __forceinline__ void buf_store(rsrc_t r, uint32_t 
 template <int AUX> __device__ __forceinline__ void buf_store(rsrc_t r, uint32_t off, const float& v)
 {
     __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned int, v), r, off, 0, AUX);
+}
+
+// ---- NHWC stack <-> NHWC tensor with buffer addressing ------------------------------------------
+//
+// The row-segment copies again, for images and blocks below 2^30 floats (everything but the largest
+// tensors; the kernels above remain for those): both sides go through range-checked descriptors, lanes
+// with nothing to move get an out-of-range offset, and there is no control flow between the first load
+// and the last store.  In the branchy version every conditional store was preceded by a full wait for
+// outstanding memory operations, stores included, so the four stores of a lane went out one after the
+// completion of the other.
+
+template <int VEC>
+__global__ __launch_bounds__(256) void k_gather_nhwc(const float* __restrict__ x, float* __restrict__ y,
+                                                     const int16_t* __restrict__ idx, NhwcArgs a)
+{
+    typedef typename Vec<VEC>::type vec;
+    const uint32_t lane = threadIdx.x & 63;
+    uint32_t unit = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (unit >= a.units) return;
+    unit = __builtin_amdgcn_readfirstlane(unit);
+    const uint32_t ib = fdiv(unit, a.dCpb);
+    if (beyond_count(a.g, ib)) return;
+    const uint32_t chunk = unit - ib * a.cpb;
+    const BlockOrigin o = origin_of(load_triple(idx, ib), a.g);
+    const int CV = a.g.C / VEC;
+    const int slo = max(0, -o.w0), shi = min(a.g.S, a.g.W - o.w0);
+    const int lo = slo * CV, hi = shi * CV;
+    const int64_t imgFloats = (int64_t)a.g.H * a.g.W * a.g.C;
+    const rsrc_t xr = make_rsrc(x + (o.valid ? (int64_t)o.n * imgFloats : 0), o.valid ? (uint32_t)imgFloats * 4u : 0u);
+    const rsrc_t yr = make_rsrc(y + (int64_t)ib * a.blockV * VEC, a.blockV * (uint32_t)(VEC * 4));
+    const uint32_t e0 = chunk * NHWC_CHUNK + lane;
+    vec v[NHWC_UNR];
+#pragma unroll
+    for (int u = 0; u < NHWC_UNR; ++u) {
+        const uint32_t e = e0 + u * 64;
+        const uint32_t r = fdiv(e, a.dRow);
+        const int j = (int)(e - r * a.rowV);
+        const int hh = o.h0 + (int)r;
+        const bool ok = e < a.blockV && (unsigned)hh < (unsigned)a.g.H && j >= lo && j < hi;
+        // (unsigned arithmetic: the value only matters when ok, and then it is the in-range offset)
+        const uint32_t off = (((uint32_t)hh * (uint32_t)a.g.W + (uint32_t)o.w0) * (uint32_t)CV + (uint32_t)j) * (uint32_t)(VEC * 4);
+        v[u] = buf_load<VEC>(xr, ok ? off : BUF_OOB);
+    }
+#pragma unroll
+    for (int u = 0; u < NHWC_UNR; ++u) {
+        const uint32_t e = e0 + u * 64;
+        buf_store<BUF_NT>(yr, e < a.blockV ? e * (uint32_t)(VEC * 4) : BUF_OOB, v[u]);
+    }
+}
+
+template <int VEC, int MODE>
+__global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ x, float* __restrict__ y,
+                                                      const int16_t* __restrict__ idx, NhwcArgs a, ColorArgs col)
+{
+    typedef typename Vec<VEC>::type vec;
+    const uint32_t lane = threadIdx.x & 63;
+    uint32_t unit = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (unit >= a.units) return;
+    unit = __builtin_amdgcn_readfirstlane(unit);
+    const uint32_t ib = fdiv(unit, a.dCpb);
+    if (beyond_count(a.g, ib)) return;
+    const uint32_t chunk = unit - ib * a.cpb;
+    const BlockOrigin o = origin_of(load_triple(idx, ib), a.g);
+    if (!o.valid) return;
+    bool atomics = MODE == SCATTER_ATOMIC;
+    if (MODE == SCATTER_COLOR && color_skip(col, o, atomics)) return;
+    const int CV = a.g.C / VEC;
+    const int slo = max(0, -o.w0), shi = min(a.g.S, a.g.W - o.w0);
+    const int lo = slo * CV, hi = shi * CV;
+    const int64_t imgFloats = (int64_t)a.g.H * a.g.W * a.g.C;
+    float* __restrict__ img = y + (int64_t)o.n * imgFloats;
+    const rsrc_t yr = make_rsrc(img, (uint32_t)imgFloats * 4u);
+    const rsrc_t xr = make_rsrc(x + (int64_t)ib * a.blockV * VEC, a.blockV * (uint32_t)(VEC * 4));
+    const uint32_t e0 = chunk * NHWC_CHUNK + lane;
+    vec v[NHWC_UNR];
+    uint32_t dst[NHWC_UNR];
+#pragma unroll
+    for (int u = 0; u < NHWC_UNR; ++u) {
+        const uint32_t e = e0 + u * 64;
+        const uint32_t r = fdiv(e, a.dRow);
+        const int j = (int)(e - r * a.rowV);
+        const int hh = o.h0 + (int)r;
+        const bool ok = e < a.blockV && (unsigned)hh < (unsigned)a.g.H && j >= lo && j < hi;
+        dst[u] = ok ? (((uint32_t)hh * (uint32_t)a.g.W + (uint32_t)o.w0) * (uint32_t)CV + (uint32_t)j) * (uint32_t)(VEC * 4)
+                    : BUF_OOB;
+        v[u] = buf_load<VEC>(xr, ok ? e * (uint32_t)(VEC * 4) : BUF_OOB);  // off-image parts are not read
+    }
+    if (MODE == SCATTER_ASSIGN) {
+#pragma unroll
+        for (int u = 0; u < NHWC_UNR; ++u) buf_store<BUF_NT>(yr, dst[u], v[u]);
+    } else if (MODE == SCATTER_ADD || (MODE == SCATTER_COLOR && !atomics)) {
+        vec cur[NHWC_UNR];
+#pragma unroll
+        for (int u = 0; u < NHWC_UNR; ++u) cur[u] = buf_load<VEC>(yr, dst[u]);
+#pragma unroll
+        for (int u = 0; u < NHWC_UNR; ++u) buf_store<BUF_NT>(yr, dst[u], vadd(cur[u], v[u]));
+    } else {
+#pragma unroll
+        for (int u = 0; u < NHWC_UNR; ++u) {
+            if (dst[u] != BUF_OOB) {
+                float* d = img + (dst[u] >> 2);
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) atomic_add_f32(d + k, vget(v[u], k));
+            }
+        }
+    }
 }
 
 // NHWC side of a tile: thread tid owns channel vector cl = tid & (lpp-1) of pixels pl0 + u*step,
@@ -1350,6 +1456,12 @@ static bool make_nhwc_args(const Geom& g, int numActive, int vec, NhwcArgs& a)
     return true;
 }
 
+// 32-bit byte offsets inside one image and inside one block: the buffer-addressed NHWC kernels apply.
+static bool nhwc_fits_buffers(const Geom& g)
+{
+    return (int64_t)g.H * g.W * g.C < (1ll << 30) && (int64_t)g.R * g.S * g.C < (1ll << 30);
+}
+
 // Chooses the tile and the workgroup size of the planar kernels; the grid is one workgroup per tile.
 static bool make_tile_args(const Geom& g, int numActive, int vec, TileArgs& a, int& threads, size_t& ldsBytes,
                            unsigned& grid, int defaultLdsBudget)
@@ -1477,7 +1589,10 @@ static void gather_dispatch(const float* x, float* y, const int16_t* idx, const 
     if (!transpose) {
         NhwcArgs a;
         if (!make_nhwc_args(g, numActive, VEC, a)) { err = hipErrorInvalidValue; return; }
-        hipLaunchKernelGGL(k_gather_nhwc<VEC>, dim3((a.units + 3) / 4), dim3(256), 0, stream, x, y, idx, a);
+        if (nhwc_fits_buffers(g))
+            hipLaunchKernelGGL(k_gather_nhwc<VEC>, dim3((a.units + 3) / 4), dim3(256), 0, stream, x, y, idx, a);
+        else
+            hipLaunchKernelGGL(k_gather_nhwc_wide<VEC>, dim3((a.units + 3) / 4), dim3(256), 0, stream, x, y, idx, a);
     } else {
         TileArgs a;
         int threads;
@@ -1531,8 +1646,12 @@ static void scatter_dispatch(const float* x, float* y, const int16_t* idx, const
     if (!transpose) {
         NhwcArgs a;
         if (!make_nhwc_args(g, numActive, VEC, a)) { err = hipErrorInvalidValue; return; }
-        hipLaunchKernelGGL((k_scatter_nhwc<VEC, MODE>), dim3((a.units + 3) / 4), dim3(256), 0, stream, x, y, idx, a,
-                           ColorArgs{1, 1, 0, nullptr});
+        if (nhwc_fits_buffers(g))
+            hipLaunchKernelGGL((k_scatter_nhwc<VEC, MODE>), dim3((a.units + 3) / 4), dim3(256), 0, stream, x, y, idx,
+                               a, ColorArgs{1, 1, 0, nullptr});
+        else
+            hipLaunchKernelGGL((k_scatter_nhwc_wide<VEC, MODE>), dim3((a.units + 3) / 4), dim3(256), 0, stream, x, y,
+                               idx, a, ColorArgs{1, 1, 0, nullptr});
     } else {
         TileArgs a;
         int threads;
@@ -1673,9 +1792,15 @@ static bool color_passes(const float* x, float* y, const int16_t* idx, const Geo
     if (!transpose) {
         NhwcArgs a;
         if (!make_nhwc_args(g, numActive, VEC, a)) return false;
-        for (col.pass = 0; col.pass < passes; ++col.pass)
-            hipLaunchKernelGGL((k_scatter_nhwc<VEC, SCATTER_COLOR>), dim3((a.units + 3) / 4), dim3(256), 0, stream, x, y,
-                               idx, a, col);
+        const bool buf = nhwc_fits_buffers(g);
+        for (col.pass = 0; col.pass < passes; ++col.pass) {
+            if (buf)
+                hipLaunchKernelGGL((k_scatter_nhwc<VEC, SCATTER_COLOR>), dim3((a.units + 3) / 4), dim3(256), 0, stream,
+                                   x, y, idx, a, col);
+            else
+                hipLaunchKernelGGL((k_scatter_nhwc_wide<VEC, SCATTER_COLOR>), dim3((a.units + 3) / 4), dim3(256), 0,
+                                   stream, x, y, idx, a, col);
+        }
     } else {
         TileArgs a;
         int threads;
