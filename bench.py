@@ -5,13 +5,18 @@
 
 A step is one pass of the path over the LiDAR-BEV-shaped workload (x = [1,800,800,128] fp32,
 27x27 blocks, stride 25, offset -1, max pooling, tol 0.5, `--density` of the 1024 blocks active):
-reduce_mask with the reference's host-visible count, sparse_gather with the fused transpose, and
-sparse_scatter_var in place (add=False, same geometry).  Inputs are resident in HBM before the timed
-region; three independent buffer sets (more than 1 GB in total) are rotated so the 256 MB Infinity
-Cache cannot serve one step's data to the next.  All calls go through the C ABI of libsbnet_amd.so
-with ctypes; PyTorch only owns the device buffers and the stream.
+reduce_mask, sparse_gather with the fused transpose, and sparse_scatter_var in place (add=False, same
+geometry).  Inputs are resident in HBM before the timed region; three independent buffer sets (more
+than 1 GB in total) are rotated so the 256 MB Infinity Cache cannot serve one step's data to the next.
+All calls go through the C ABI of libsbnet_amd.so with ctypes; PyTorch only owns the device buffers
+and the stream.
 
-One JSON line goes to stdout.  `value` is algorithmic bytes per step / wall time per step.  `ops`
+The step is timed three ways (`pipeline` in the output): with the reference's host-visible count
+(reduce_mask waits for a 4-byte copy, the host sizes the other launches), with the count left on the
+device (the `_device_count` entry points, three calls per step), and with those three launches captured
+in a HIP graph and replayed.  One JSON line goes to stdout.  `value` is algorithmic bytes per step /
+wall time per step with the count on the device (eager launches); the other two are reported beside
+it.  `ops`
 holds per-op device times (HIP events around batches of back-to-back launches on the launch stream),
 `roofline` the dominant kernel (the transposing gather) against the 8 TB/s HBM peak, `cpu_baseline`
 the single-threaded CPU oracle (the reference's CPU functors restated; the reference builds them
@@ -329,33 +334,64 @@ def main():
     wl = workloads.config3(args.density)
     path = Path(wl, torch, lib, nsets=3)
     nsets = len(path.sets)
-    for i in range(args.warmup):
-        path.step(i % nsets)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        M = path.step(i % nsets)
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    assert M == path.M, "active block count changed between runs"
-    ms_per_step = wall / args.steps * 1e3
     step_bytes = sum(path.bytes.values())
-    value = step_bytes / (ms_per_step * 1e-3) * 1e-9
 
-    # the same pipeline without the host-visible count (not the reference's contract; reported beside `value`)
-    for i in range(max(args.warmup, nsets)):
-        path.step_device_count(i % nsets)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        path.step_device_count(i % nsets)
-    torch.cuda.synchronize()
-    dc_ms = (time.perf_counter() - t0) / args.steps * 1e3
+    def timed(step_fn):
+        """W untimed steps, then exactly K steps between two device synchronisations; ms per step."""
+        for i in range(max(args.warmup, nsets)):
+            step_fn(i % nsets)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            step_fn(i % nsets)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / args.steps * 1e3
+
+    def variant(ms, note):
+        return {"ms_per_step": round(ms, 4), "GBps": round(step_bytes / (ms * 1e-3) * 1e-9, 1), "note": note}
+
+    # (1) the reference's contract: reduce_mask hands the count to the host, which sizes the other two launches
+    counts = []
+    host_ms = timed(lambda i: counts.append(path.step(i)))
+    assert counts[-1] == path.M, "active block count changed between runs"
+
+    # (2) the count stays on the device: launches sized for max_active blocks, nothing waits for the host
+    dc_ms = timed(path.step_device_count)
     dc_counts = [int(s["dcount"].cpu()[0]) for s in path.sets]
     assert dc_counts == [path.M] * nsets, "device-resident count differs from the host-visible one"
+
+    # (3) the same three launches captured once per buffer set into a HIP graph and replayed
+    eager_stream = path.stream
+    graphs = []
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        path.stream = ctypes.c_void_p(side.cuda_stream)
+        for i in range(nsets):
+            path.step_device_count(i)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    for i in range(nsets):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            path.stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            path.step_device_count(i)
+        graphs.append(g)
+    path.stream = eager_stream
+    for s in path.sets:
+        s["dcount"].zero_()
+    graph_ms = timed(lambda i: graphs[i].replay())
+    dc_counts = [int(s["dcount"].cpu()[0]) for s in path.sets]
+    assert dc_counts == [path.M] * nsets, "graph replay produced a different count"
+    del graphs
     for s in path.sets:
         s.pop("stack_cap", None)
     torch.cuda.empty_cache()
+
+    # `value`: the pipeline as this library is meant to be driven (count on the device, nothing waits for the
+    # host).  The reference's host-count contract and the graph replay are reported beside it.
+    ms_per_step = dc_ms
+    value = step_bytes / (ms_per_step * 1e-3) * 1e-9
 
     ops = path.op_table()
     g = ops["gather"]
@@ -365,7 +401,7 @@ def main():
                 "algorithmic_bytes_per_launch": g["bytes"],
                 "traffic": read_measured_traffic("gather_planar_C3_pmc.txt")}
     out = {
-        "metric": "achieved HBM GB/s over reduce_mask+sparse_gather+sparse_scatter_var (algorithmic bytes / wall time per step)",
+        "metric": "achieved HBM GB/s over reduce_mask+sparse_gather+sparse_scatter_var (algorithmic bytes / wall time per step); us/op and % of HBM peak under ops and roofline",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
@@ -374,11 +410,15 @@ def main():
                                % (round(args.density * 100), path.M),
                    "buffer_sets": nsets, "bytes_per_step": step_bytes},
         "ops": ops, "roofline": roofline,
-        "pipeline_device_count": {"ms_per_step": round(dc_ms, 4),
-                                  "GBps": round(step_bytes / (dc_ms * 1e-3) * 1e-9, 1),
-                                  "max_active": path.maxidx,
-                                  "note": "count read on the device, launches sized for max_active blocks, "
-                                          "no host sync inside a step"},
+        "pipeline": {
+            "device_count_graph": variant(graph_ms, "count read on the device, reduce_mask + gather + scatter_var "
+                                                    "captured in one HIP graph per buffer set, one replay per step"),
+            "device_count_eager": variant(dc_ms, "value: count read on the device, three C-ABI calls per step from Python, "
+                                                 "launches sized for max_active=%d blocks" % path.maxidx),
+            "host_count_reference_contract": variant(host_ms, "reduce_mask copies the count to the host and waits "
+                                                              "(the reference's HostMemory output), gather and "
+                                                              "scatter sized from it"),
+        },
     }
     if not args.no_cpu:
         nb = path.bytes["gather"] + path.bytes["scatter"]

@@ -359,6 +359,7 @@ struct TileArgs {
     int cchunks;        // channel chunks per block
     uint32_t tpb;       // tiles per block = psplit * cchunks
     uint32_t total;     // numActive * tpb
+    int grid2d;         // the launch is (tpb, numActive): the block is blockIdx.y and needs no division
     uint32_t vpr;       // slots per planar row: (P + 3) / 4
     int64_t imgFloats;  // H * W * C
     uint32_t imgBytes;  // H * W * C * 4, below 2^32 (the host falls back to k_planar_small otherwise)
@@ -370,10 +371,18 @@ struct TileId {
     int c0, ctEff, p0, Pn;
 };
 
-__device__ __forceinline__ void decode_tile(const TileArgs& a, uint32_t id, TileId& t)
+// With a (tiles per block, blocks) launch the block number comes straight from the workgroup id, so the load
+// of its index triple can be issued from preloaded kernel arguments before anything else arrives.
+__device__ __forceinline__ void decode_tile(const TileArgs& a, TileId& t)
 {
-    t.ib = fdiv(id, a.dTpb);
-    const uint32_t rem = id - t.ib * a.tpb;
+    uint32_t rem;
+    if (a.grid2d) {
+        t.ib = blockIdx.y;
+        rem = blockIdx.x;
+    } else {
+        t.ib = fdiv(blockIdx.x, a.dTpb);
+        rem = blockIdx.x - t.ib * a.tpb;
+    }
     const uint32_t cc = fdiv(rem, a.dPs);
     const uint32_t pc = rem - cc * (uint32_t)a.psplit;
     t.c0 = (int)cc * a.Ct;
@@ -589,9 +598,10 @@ __global__ __launch_bounds__(512) void k_gather_planar(const float* __restrict__
     const uint32_t tid = threadIdx.x, nthr = blockDim.x;
     const uint32_t RS = (uint32_t)(a.g.R * a.g.S);
     TileId t;
-    decode_tile(a, blockIdx.x, t);
+    decode_tile(a, t);
+    const RawTriple raw = load_triple(idx, t.ib);
     if (beyond_count(a.g, t.ib)) return;
-    const BlockOrigin o = origin_of(load_triple(idx, t.ib), a.g);
+    const BlockOrigin o = origin_of(raw, a.g);
     // a block index outside [0, N) gets an empty descriptor: every load returns 0
     const rsrc_t xr = make_rsrc(x + (o.valid ? (int64_t)o.n * a.imgFloats : 0), o.valid ? a.imgBytes : 0u);
 
@@ -681,7 +691,7 @@ struct LineArgs {
     int RS;
     int P, Pp, psplit, cchunks;
     int ext;            // window pixels beyond the tile's own: LINE_EXT
-    int xcd;            // > 0: tiles of one chunk are spread over workgroup ids xcd apart
+    int grid2d;         // the launch is (tpb, numActive): the block is blockIdx.y
     uint32_t tpb, total;
     uint32_t spr;       // bound on the output slots of one row of one tile
     int64_t imgFloats;
@@ -697,21 +707,16 @@ __global__ __launch_bounds__(512) void k_gather_lines(const float* __restrict__ 
     const uint32_t tid = threadIdx.x, nthr = blockDim.x;
     const uint32_t RS = (uint32_t)a.RS;
 
-    // tile id.  Consecutive workgroup ids go to different XCDs (each with its own L2); with xcd set, the
-    // splits of one chunk, whose windows overlap, get ids that are xcd apart and so share an L2.
-    uint32_t id = blockIdx.x;
-    if (a.xcd > 0) {
-        const uint32_t group = (uint32_t)a.xcd * (uint32_t)a.psplit;
-        const uint32_t full = a.total / group * group;
-        if (id < full) {
-            const uint32_t gidx = id / group, r = id - gidx * group;
-            const uint32_t lane = r % (uint32_t)a.xcd, split = r / (uint32_t)a.xcd;
-            id = (gidx * (uint32_t)a.xcd + lane) * (uint32_t)a.psplit + split;
-        }
+    uint32_t ib, rem;
+    if (a.grid2d) {
+        ib = blockIdx.y;
+        rem = blockIdx.x;
+    } else {
+        ib = fdiv(blockIdx.x, a.dTpb);
+        rem = blockIdx.x - ib * a.tpb;
     }
-    const uint32_t ib = fdiv(id, a.dTpb);
+    const RawTriple raw = load_triple(idx, ib);
     if (beyond_count(a.g, ib)) return;
-    const uint32_t rem = id - ib * a.tpb;
     const uint32_t cc = fdiv(rem, a.dPs);
     const uint32_t split = rem - cc * (uint32_t)a.psplit;
     const uint32_t c0 = cc * (uint32_t)a.Ct;
@@ -720,7 +725,7 @@ __global__ __launch_bounds__(512) void k_gather_lines(const float* __restrict__ 
     const uint32_t p1 = min(p0 + (uint32_t)a.P, RS);
     const uint32_t win = p1 - p0 + (uint32_t)a.ext;
 
-    const BlockOrigin o = origin_of(load_triple(idx, ib), a.g);
+    const BlockOrigin o = origin_of(raw, a.g);
     const rsrc_t xr = make_rsrc(x + (o.valid ? (int64_t)o.n * a.imgFloats : 0), o.valid ? a.imgBytes : 0u);
 
     // NHWC side: lane owns channels [4*cl, 4*cl + 4) of window pixels q0 + u*step.  (r, s) of the pixel is
@@ -848,9 +853,9 @@ __global__ __launch_bounds__(512) void k_scatter_planar(const float* __restrict_
     const uint32_t tid = threadIdx.x, nthr = blockDim.x;
     const uint32_t RS = (uint32_t)(a.g.R * a.g.S);
     TileId t;
-    decode_tile(a, blockIdx.x, t);
-    if (beyond_count(a.g, t.ib)) return;
+    decode_tile(a, t);
     const RawTriple raw = load_triple(idx, t.ib);  // scalar load, needed only after the barrier
+    if (beyond_count(a.g, t.ib)) return;
     bool atomics = MODE == SCATTER_ATOMIC;
     if (MODE == SCATTER_COLOR && color_skip(col, origin_of(raw, a.g), atomics)) return;  // (here: before the loads)
 
@@ -1354,9 +1359,17 @@ static uint32_t pow2_ceil(uint32_t v)
     return p;
 }
 
-// Optional overrides for experiments: SBNET_TUNE="ct=32,lds=32768,wg=256,ps=3,xcd=8,lines=1".
+constexpr int GRID_Y_MAX = 65535;
+
+// One workgroup per tile, as (tiles per block, blocks) when the block count fits the y dimension of a launch.
+static dim3 tile_grid(int grid2d, uint32_t tpb, int numActive, uint32_t total)
+{
+    return grid2d ? dim3(tpb, (unsigned)numActive) : dim3(total);
+}
+
+// Optional overrides for experiments: SBNET_TUNE="ct=32,lds=32768,wg=256,ps=3,lines=1".
 struct Tune {
-    int ct = 0, ldsBytes = 0, wg = 0, ps = 0, xcd = -1, lines = -1;
+    int ct = 0, ldsBytes = 0, wg = 0, ps = 0, lines = -1, pad = 0;
 };
 
 static Tune read_tune()
@@ -1369,8 +1382,8 @@ static Tune read_tune()
     if ((p = strstr(s, "lds="))) t.ldsBytes = atoi(p + 4);
     if ((p = strstr(s, "wg="))) t.wg = atoi(p + 3);
     if ((p = strstr(s, "ps="))) t.ps = atoi(p + 3);
-    if ((p = strstr(s, "xcd="))) t.xcd = atoi(p + 4);
     if ((p = strstr(s, "lines="))) t.lines = atoi(p + 6);
+    if ((p = strstr(s, "pad="))) t.pad = atoi(p + 4);
     return t;
 }
 
@@ -1514,6 +1527,7 @@ static bool make_tile_args(const Geom& g, int numActive, int vec, TileArgs& a, i
     ldsBytes = (size_t)a.Ct * a.Pp * sizeof(float);
     if (ldsBytes > 64 * 1024) return false;
     grid = a.total;
+    a.grid2d = numActive <= GRID_Y_MAX;
     return true;
 }
 
@@ -1552,6 +1566,7 @@ static bool make_line_args(const Geom& g, int numActive, const float* y, LineArg
         a.psplit = (RS + cap - 1) / cap;
     }
     if (tune.ps > 0) a.psplit = tune.ps;
+    if (tune.wg > 0) threads = tune.wg;
     a.P = (RS + a.psplit - 1) / a.psplit;
     a.psplit = (RS + a.P - 1) / a.P;
     // A tile that takes whole planes writes one contiguous piece of y in k_gather_planar already.
@@ -1563,7 +1578,7 @@ static bool make_line_args(const Geom& g, int numActive, const float* y, LineArg
     if (ld < 4) ld = 4;
     if (ld > 8) return false;
     a.Pp = (win + 3 + 31) / 32 * 32;
-    ldsBytes = (size_t)a.Ct * a.Pp * sizeof(float);
+    ldsBytes = (size_t)a.Ct * a.Pp * sizeof(float) + (size_t)tune.pad;
     if (ldsBytes > 64 * 1024) return false;
     // slots per row: the written range of a row is at most P + LINE_EXT floats; when every chunk starts on a
     // line it is a whole number of lines
@@ -1574,11 +1589,11 @@ static bool make_line_args(const Geom& g, int numActive, const float* y, LineArg
     const uint64_t total = (uint64_t)numActive * a.tpb;
     if (total >= (1ull << 31)) return false;
     a.total = (uint32_t)total;
-    a.xcd = tune.xcd >= 0 ? tune.xcd : 0;
     a.dTpb = make_fastdiv(a.tpb);
     a.dPs = make_fastdiv((uint32_t)a.psplit);
     a.dS = make_fastdiv((uint32_t)g.S);
     grid = a.total;
+    a.grid2d = numActive <= GRID_Y_MAX;
     return true;
 }
 
@@ -1602,12 +1617,13 @@ static void gather_dispatch(const float* x, float* y, const int16_t* idx, const 
             LineArgs la;
             int ld;
             if (make_line_args(g, numActive, y, la, threads, ld, lds, grid)) {
+                const dim3 lg = tile_grid(la.grid2d, la.tpb, numActive, la.total);
                 switch (ld) {
-                case 4: hipLaunchKernelGGL(k_gather_lines<4>, dim3(grid), dim3(threads), lds, stream, x, y, idx, la); break;
-                case 5: hipLaunchKernelGGL(k_gather_lines<5>, dim3(grid), dim3(threads), lds, stream, x, y, idx, la); break;
-                case 6: hipLaunchKernelGGL(k_gather_lines<6>, dim3(grid), dim3(threads), lds, stream, x, y, idx, la); break;
-                case 7: hipLaunchKernelGGL(k_gather_lines<7>, dim3(grid), dim3(threads), lds, stream, x, y, idx, la); break;
-                default: hipLaunchKernelGGL(k_gather_lines<8>, dim3(grid), dim3(threads), lds, stream, x, y, idx, la); break;
+                case 4: hipLaunchKernelGGL(k_gather_lines<4>, lg, dim3(threads), lds, stream, x, y, idx, la); break;
+                case 5: hipLaunchKernelGGL(k_gather_lines<5>, lg, dim3(threads), lds, stream, x, y, idx, la); break;
+                case 6: hipLaunchKernelGGL(k_gather_lines<6>, lg, dim3(threads), lds, stream, x, y, idx, la); break;
+                case 7: hipLaunchKernelGGL(k_gather_lines<7>, lg, dim3(threads), lds, stream, x, y, idx, la); break;
+                default: hipLaunchKernelGGL(k_gather_lines<8>, lg, dim3(threads), lds, stream, x, y, idx, la); break;
                 }
                 return;
             }
@@ -1621,7 +1637,8 @@ static void gather_dispatch(const float* x, float* y, const int16_t* idx, const 
                                dim3(256), 0, stream, x, y, idx, g, total);
             return;
         }
-        hipLaunchKernelGGL(k_gather_planar<VEC>, dim3(grid), dim3(threads), lds, stream, x, y, idx, a);
+        hipLaunchKernelGGL(k_gather_planar<VEC>, tile_grid(a.grid2d, a.tpb, numActive, a.total), dim3(threads), lds,
+                           stream, x, y, idx, a);
     }
 }
 
@@ -1665,8 +1682,8 @@ static void scatter_dispatch(const float* x, float* y, const int16_t* idx, const
                                0, stream, x, y, idx, g, total);
             return;
         }
-        hipLaunchKernelGGL((k_scatter_planar<VEC, MODE>), dim3(grid), dim3(threads), lds, stream, x, y, idx, a,
-                           ColorArgs{1, 1, 0, nullptr});
+        hipLaunchKernelGGL((k_scatter_planar<VEC, MODE>), tile_grid(a.grid2d, a.tpb, numActive, a.total), dim3(threads),
+                           lds, stream, x, y, idx, a, ColorArgs{1, 1, 0, nullptr});
     }
 }
 
@@ -1808,8 +1825,8 @@ static bool color_passes(const float* x, float* y, const int16_t* idx, const Geo
         unsigned grid;
         if ((int64_t)g.R * g.S < 4 || !make_tile_args(g, numActive, VEC, a, threads, lds, grid, 16 * 1024)) return false;
         for (col.pass = 0; col.pass < passes; ++col.pass)
-            hipLaunchKernelGGL((k_scatter_planar<VEC, SCATTER_COLOR>), dim3(grid), dim3(threads), lds, stream, x, y, idx,
-                               a, col);
+            hipLaunchKernelGGL((k_scatter_planar<VEC, SCATTER_COLOR>), tile_grid(a.grid2d, a.tpb, numActive, a.total),
+                               dim3(threads), lds, stream, x, y, idx, a, col);
     }
     return true;
 }

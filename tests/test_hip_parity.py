@@ -369,6 +369,29 @@ def test_reduce_mask_many_blocks_and_async_count():
     np.testing.assert_array_equal(host(r2.active_block_indices)[:int(cnt_o[0])], idx_o[:int(cnt_o[0])])
 
 
+@pytest.mark.parametrize("bs,bst,bo", [((2, 2), (2, 2), (0, 0)), ((3, 3), (2, 2), (-1, -1))])
+def test_more_blocks_than_a_launch_dimension_holds(bs, bst, bo):
+    """More than 65 535 active blocks: the planar kernels then number their workgroups along one launch
+    dimension instead of (tiles, blocks).  Whole pipeline, both stack layouts."""
+    rng = np.random.default_rng(21)
+    N, H, W, C = 1200, 16, 16, 8
+    mask = (rng.random((N, H, W, 1)) < 0.97).astype(np.float32)
+    x = rng.standard_normal((N, H, W, C)).astype(np.float32)
+    bc = [8, 8]
+    idx_o, cnt_o, r = check_reduce(mask, bc, bs, bst, bo, 0.5, False)
+    assert int(cnt_o[0]) > 65535
+    xd = dev(x)
+    for transpose in (False, True):
+        g_o = orc.sparse_gather(x, cnt_o, idx_o, bs, bst, bo, transpose=transpose)
+        g = sbnet_amd.sparse_gather(xd, r.bin_counts, r.active_block_indices, bs, bst, bo, transpose=transpose)
+        np.testing.assert_array_equal(host(g), g_o)
+        base = np.full_like(x, 3.0)
+        y_o = orc.sparse_scatter(g_o, cnt_o, idx_o, base, bs, bst, bo, add=False, transpose=transpose)
+        y = sbnet_amd.sparse_scatter_var(g, r.bin_counts, r.active_block_indices, dev(base), bs, bst, bo, add=False,
+                                         transpose=transpose)
+        np.testing.assert_array_equal(host(y), y_o)
+
+
 def test_reduce_mask_rows_past_count_untouched():
     mask = np.zeros((1, 8, 8, 1), np.float32)
     mask[0, 0, 0, 0] = 1.0
