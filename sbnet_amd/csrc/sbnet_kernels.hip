@@ -990,7 +990,7 @@ struct PoolArgs {
     uint32_t T;       // N * bCntH * bCntW
     float tol;
     int avg;
-    int logG, logGw;  // lanes per block, lanes along w inside a group
+    int logG;         // log2 of the lanes that share one block
     int passes;       // blocks per group
     FastDiv dBw, dBhw;
 };
@@ -1006,6 +1006,8 @@ __device__ __forceinline__ float next_down(float f)
 
 __device__ __forceinline__ float next_up(float f) { return -next_down(-f); }
 
+constexpr int POOL_LD = 8;  // loads in flight per lane
+
 __global__ __launch_bounds__(256) void k_reduce_pool(const float* __restrict__ mask, PoolArgs a,
                                                      uint8_t* __restrict__ flags, int32_t* __restrict__ counts)
 {
@@ -1014,11 +1016,10 @@ __global__ __launch_bounds__(256) void k_reduce_pool(const float* __restrict__ m
     if (tid == 0) wgCount = 0;
     __syncthreads();
 
-    const int G = 1 << a.logG, Gw = 1 << a.logGw, Gh = G >> a.logGw;
+    const int G = 1 << a.logG;
     const uint32_t groups = 256u >> a.logG;
     const uint32_t grp = tid >> a.logG;
     const int l = (int)(tid & (uint32_t)(G - 1));
-    const int lc = l & (Gw - 1), lr = l >> a.logGw;
     const uint32_t CH = groups * (uint32_t)a.passes;
     const float denom = (float)(a.R * a.S);
 
@@ -1038,16 +1039,38 @@ __global__ __launch_bounds__(256) void k_reduce_pool(const float* __restrict__ m
         const float* __restrict__ img = mask + (int64_t)n * a.H * a.W;
         float sum = 0.f, sabs = 0.f;
         int allint = 1, any = 0;
-        for (int hh = hlo + lr; hh < hhi; hh += Gh) {
-            const float* __restrict__ row = img + (int64_t)hh * a.W;
-            for (int ww = wlo + lc; ww < whi; ww += Gw) {
-                const float v = row[ww];
+        // The clipped window, flattened row-major, is dealt to the G lanes in turn; POOL_LD loads per lane go
+        // out back to back before the first one is used (the window is a handful of cache lines per lane, so
+        // the kernel is a chain of load latencies and nothing else).  Lanes past the end read element 0 of
+        // the window's first row, which exists whenever the window is not empty.
+        const uint32_t cw = (uint32_t)max(0, whi - wlo), chh = (uint32_t)max(0, hhi - hlo);
+        const uint32_t npxc = cw * chh;  // below 2^31: the host checks R*S
+        const float* __restrict__ win = img + (int64_t)hlo * a.W + wlo;
+        const uint32_t stepR = (uint32_t)G / max(cw, 1u), stepS = (uint32_t)G - stepR * cw;
+        uint32_t r = (uint32_t)l / max(cw, 1u), sc = (uint32_t)l - r * cw;
+        for (uint32_t e0 = (uint32_t)l; e0 < npxc; e0 += POOL_LD * (uint32_t)G) {
+            float v[POOL_LD];
+            bool ok[POOL_LD];
+#pragma unroll
+            for (int k = 0; k < POOL_LD; ++k) {
+                ok[k] = e0 + (uint32_t)k * (uint32_t)G < npxc;
+                v[k] = win[ok[k] ? (int64_t)r * a.W + sc : 0];
+                sc += stepS;
+                r += stepR;
+                if (sc >= cw) {
+                    sc -= cw;
+                    ++r;
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < POOL_LD; ++k) {
                 if (a.avg) {
-                    sum += v;
-                    sabs += fabsf(v);
-                    allint &= (v == truncf(v));
+                    const float t = ok[k] ? v[k] : 0.f;
+                    sum += t;
+                    sabs += fabsf(t);
+                    allint &= (t == truncf(t));
                 } else {
-                    any |= (v > a.tol);
+                    any |= (ok[k] && v[k] > a.tol);
                 }
             }
         }
@@ -1420,11 +1443,11 @@ hipError_t launch_reduce_mask(const float* mask, const Geom& g, int bCntH, int b
     p.tol = tol;
     p.avg = avgPool ? 1 : 0;
     const uint64_t npx = (uint64_t)g.R * (uint64_t)g.S;
+    // the kernel counts the pixels of a block's in-image window in 32 bits
+    if ((uint64_t)(g.R < g.H ? g.R : g.H) * (uint64_t)(g.S < g.W ? g.S : g.W) >= (1ull << 31)) return hipErrorInvalidValue;
     int logG = npx >= 16 ? ilog2_floor((uint32_t)(npx / 8 > 64 ? 64 : npx / 8)) : 0;
     if (logG > 6) logG = 6;
     p.logG = logG;
-    const uint32_t Gw = pow2_ceil((uint32_t)g.S);
-    p.logGw = ilog2_floor(Gw < (1u << logG) ? Gw : (1u << logG));
     const uint32_t groups = 256u >> logG;
     int passes = 1;
     while (passes < (1 << logG) && passes < 8 && T / (groups * passes) > 2048) passes *= 2;
