@@ -267,7 +267,7 @@ def cpu_baseline(wl, M, idx_host, nbytes, budget_s=12.0):
 
     run(False)
     times, spent = [], 0.0
-    while spent < budget_s * 0.7 and len(times) < 40:
+    while spent < budget_s * 0.7 and len(times) < 400:
         t = run(False)
         times.append(t)
         spent += t
@@ -276,7 +276,7 @@ def cpu_baseline(wl, M, idx_host, nbytes, budget_s=12.0):
     omp_threads = int(os.environ.get("OMP_NUM_THREADS", cores))
     run(True)
     times_omp, spent = [], 0.0
-    while spent < budget_s * 0.3 and len(times_omp) < 40:
+    while spent < budget_s * 0.3 and len(times_omp) < 400:
         t = run(True)
         times_omp.append(t)
         spent += t
@@ -399,7 +399,7 @@ def main():
                 "achieved": g["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(g["GBps"] / HBM_PEAK_GBS, 4), "us_per_launch": g["us"],
                 "algorithmic_bytes_per_launch": g["bytes"],
-                "traffic": read_measured_traffic("gather_planar_C3_pmc.txt")}
+                "traffic": read_measured_traffic("gather_lines_scatter_planar_C3_30pct_pmc.txt")}
     out = {
         "metric": "achieved HBM GB/s over reduce_mask+sparse_gather+sparse_scatter_var (algorithmic bytes / wall time per step); us/op and % of HBM peak under ops and roofline",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

@@ -392,6 +392,35 @@ def test_more_blocks_than_a_launch_dimension_holds(bs, bst, bo):
         np.testing.assert_array_equal(host(y), y_o)
 
 
+def test_image_of_2_pow_30_floats_takes_the_64_bit_offset_kernels():
+    """An image of 2^30 floats (4 GiB) is the first size whose byte offsets do not fit 32 bits: gather and
+    scatter then leave the buffer-addressed kernels for the ones with 64-bit addressing (NHWC stack) and the
+    one-thread-per-element kernel (planar stack).  Blocks at the far end of the image, where offsets exceed
+    2^32, against the oracle; in-place scatter checked on the whole 4 GiB tensor."""
+    N, H, W, C = 1, 8192, 8192, 16
+    bs, bst, bo = (5, 6), (6, 7), (-1, -2)
+    g = torch.Generator(device=DEV).manual_seed(5)
+    xd = torch.randint(-1000, 1000, (N, H, W, C), generator=g, device=DEV, dtype=torch.int32).to(torch.float32)
+    x = host(xd)
+    bh_max, bw_max = (H - bo[0] - 1) // bst[0], (W - bo[1] - 1) // bst[1]
+    idx = np.array([[0, 0, 0], [0, bh_max, bw_max], [0, bh_max, 0], [0, bh_max - 1, bw_max - 3], [0, 1500, 77],
+                    [0, bh_max // 2 + 1, bw_max], [0, 0, bw_max]], np.int16)
+    cnt = np.array([len(idx)], np.int32)
+    idx_d, cnt_t = dev(idx), torch.from_numpy(cnt)
+    for transpose in (False, True):
+        g_o = orc.sparse_gather(x, cnt, idx, bs, bst, bo, transpose=transpose)
+        gd = sbnet_amd.sparse_gather(xd, cnt_t, idx_d, bs, bst, bo, transpose=transpose)
+        np.testing.assert_array_equal(host(gd), g_o)
+        stack = (g_o * 0.5 + 1.0).astype(np.float32)
+        y_o = orc.sparse_scatter_var(stack, cnt, idx, x.copy(), bs, bst, bo, add=True, transpose=transpose)
+        yd = xd.clone()
+        sbnet_amd.sparse_scatter_var(dev(stack), cnt_t, idx_d, yd, bs, bst, bo, add=True, transpose=transpose)
+        assert torch.equal(yd, dev(y_o))
+        del yd, y_o
+    del xd, x
+    torch.cuda.empty_cache()
+
+
 def test_reduce_mask_rows_past_count_untouched():
     mask = np.zeros((1, 8, 8, 1), np.float32)
     mask[0, 0, 0, 0] = 1.0
@@ -644,7 +673,7 @@ def test_whole_pipeline_in_a_hip_graph():
         np.testing.assert_array_equal(host(y_s), y_o)
 
 
-@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("seed", range(32))
 def test_random_geometries(seed):
     """Seeded random block geometries (sizes, strides, offsets on either side of zero, channel counts of every
     vector width, partial channel chunks, planes from 1 to ~1200 pixels), random block lists in random order
