@@ -12,7 +12,7 @@ All calls go through the C ABI of libsbnet_amd.so with ctypes; PyTorch only owns
 and the stream.
 
 The step is timed three ways (`pipeline` in the output): with the reference's host-visible count
-(reduce_mask waits for a 4-byte copy, the host sizes the other launches), with the count left on the
+(reduce_mask returns once the count has reached the host, which sizes the other launches), with the count left on the
 device (the `_device_count` entry points, three calls per step), and with those three launches captured
 in a HIP graph and replayed.  One JSON line goes to stdout.  `value` is algorithmic bytes per step /
 wall time per step with the count on the device (eager launches); the other two are reported beside
@@ -415,9 +415,10 @@ def main():
                                                     "captured in one HIP graph per buffer set, one replay per step"),
             "device_count_eager": variant(dc_ms, "value: count read on the device, three C-ABI calls per step from Python, "
                                                  "launches sized for max_active=%d blocks" % path.maxidx),
-            "host_count_reference_contract": variant(host_ms, "reduce_mask copies the count to the host and waits "
-                                                              "(the reference's HostMemory output), gather and "
-                                                              "scatter sized from it"),
+            "host_count_reference_contract": variant(host_ms, "reduce_mask returns with the count on the host "
+                                                              "(the reference's HostMemory output; stored into "
+                                                              "pinned memory by the kernel and polled), gather "
+                                                              "and scatter sized from it"),
         },
     }
     if not args.no_cpu:

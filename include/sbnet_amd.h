@@ -83,9 +83,15 @@ size_t sbnet_reduce_mask_workspace_bytes(int N, const int32_t* bcount, int bcoun
  *                         CPU functor's lexicographic (n, bh, bw) order.  Rows past the count
  *                         are left untouched.
  *   bin_counts_host       host int32[1] or NULL.  Non-NULL keeps the reference's HostMemory
- *                         contract (reduce_mask.cc:198-220): the count is copied back and the
- *                         call returns after the stream has drained.  NULL: nothing is copied,
- *                         the call is asynchronous.
+ *                         contract (reduce_mask.cc:198-220): the call returns once the count is
+ *                         in *bin_counts_host.  The kernel that knows the count stores it into a
+ *                         word of pinned host memory (one per calling thread and device, allocated
+ *                         on first use) which the call polls, so there is no device-to-host copy
+ *                         and no stream synchronisation; active_block_indices is complete in stream
+ *                         order, like any other output.  Where that word cannot be had, the count
+ *                         is copied and the stream synchronised as the reference does.  Not
+ *                         available while `stream` is being captured into a graph (SBNET_EHIP).
+ *                         NULL: nothing reaches the host, the call is asynchronous.
  *   bin_counts_device     device int32[1] or NULL; receives the same count.  At least one of
  *                         the two count pointers must be non-NULL.
  *   A mask with no active block reports count 1 and writes the triple (0,0,0)

@@ -30,6 +30,69 @@ int hip_fail(hipError_t e)
 
 bool pair_ok(const int32_t* p, int len) { return p != nullptr && len == 2; }
 
+// The host-visible count of reduce_mask (reduce_mask.cc:198-204: a HostMemory output filled by a blocking
+// cudaMemcpy).  Instead of a device-to-host copy and a stream synchronisation (about 17 us of a 113 us
+// pipeline step), the kernel that knows the count stores it, tagged with a sequence number, into one word
+// of pinned host memory and the calling thread polls that word.  One word per thread and device, allocated
+// on first use and kept until the process ends.
+constexpr int MAX_SIGNAL_DEVICES = 64;
+struct HostSignal {
+    unsigned long long* host = nullptr;  // pinned, device-visible (same address on both sides)
+    uint32_t seq = 0;
+    bool failed = false;                 // allocation refused once: do not try again
+};
+thread_local HostSignal t_signal[MAX_SIGNAL_DEVICES];
+
+HostSignal* host_signal()
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_SIGNAL_DEVICES) return nullptr;
+    HostSignal& s = t_signal[dev];
+    if (!s.host && !s.failed) {
+        void* p = nullptr;
+        if (hipHostMalloc(&p, 64, hipHostMallocMapped) != hipSuccess || !p) {
+            (void)hipGetLastError();
+            s.failed = true;
+        } else {
+            s.host = static_cast<unsigned long long*>(p);
+            *s.host = 0;
+        }
+    }
+    return s.host ? &s : nullptr;
+}
+
+// Waits until the word carries `seq` and returns the count; gives up (false) as soon as the stream has
+// drained without the word arriving or reports an error, so the wait always ends with the stream.
+bool poll_host_signal(const HostSignal& s, uint32_t seq, hipStream_t stream, int32_t* count, hipError_t* err)
+{
+    *err = hipSuccess;
+    for (uint32_t spins = 1;; ++spins) {
+        const unsigned long long v = __atomic_load_n(s.host, __ATOMIC_ACQUIRE);
+        if ((uint32_t)(v >> 32) == seq) {
+            *count = (int32_t)(uint32_t)v;
+            return true;
+        }
+        if ((spins & 255u) == 0) {
+            const hipError_t q = hipStreamQuery(stream);
+            if (q == hipErrorNotReady) {
+                (void)hipGetLastError();
+                continue;
+            }
+            if (q != hipSuccess) {
+                *err = q;
+                return false;
+            }
+            // the stream is idle: the store has been issued; look once more, then leave it to a copy
+            const unsigned long long w = __atomic_load_n(s.host, __ATOMIC_ACQUIRE);
+            if ((uint32_t)(w >> 32) == seq) {
+                *count = (int32_t)(uint32_t)w;
+                return true;
+            }
+            return false;
+        }
+    }
+}
+
 // Limits the reference leaves unchecked.  Indices are int16 triples, so n, bh and bw must fit.
 bool geom_ok(int N, int H, int W, int C, const int32_t* bsize, const int32_t* bstride)
 {
@@ -84,9 +147,30 @@ int reduce_mask_impl(const float* mask, int N, int H, int W, const int32_t* bcou
         ownWs = true;
     }
     const sbnet::Geom g = make_geom(N, H, W, 1, bsize, bstride, boffset);
+    // a host-visible count cannot be produced while the stream is being captured (nothing runs): refuse before
+    // anything is enqueued, so the capture stays valid
+    HostSignal* sig = nullptr;
+    uint32_t seq = 0;
+    if (countHost) {
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &cap) != hipSuccess) {
+            (void)hipGetLastError();
+        } else if (cap != hipStreamCaptureStatusNone) {
+            if (ownWs) (void)hipFree(ws);
+            return hip_fail(hipErrorStreamCaptureUnsupported);
+        } else {
+            sig = host_signal();
+        }
+        if (sig) {
+            seq = ++sig->seq;
+            if (seq == 0) seq = ++sig->seq;  // 0 is the word's initial tag
+        }
+    }
     hipError_t e = sbnet::launch_reduce_mask(mask, g, bcount[0], bcount[1], tol, avgpool != 0, fixup, idx,
-                                             countDev, ws, stream);
-    if (e == hipSuccess && countHost) {
+                                             countDev, ws, stream, sig ? sig->host : nullptr, seq);
+    bool haveCount = false;
+    if (e == hipSuccess && sig) haveCount = poll_host_signal(*sig, seq, stream, countHost, &e);
+    if (e == hipSuccess && countHost && !haveCount) {
         // the count sits in countDev, or behind the flags and counts of the workspace
         const int32_t* src = countDev;
         if (!src) {

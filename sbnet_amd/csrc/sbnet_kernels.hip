@@ -1129,7 +1129,8 @@ struct CompactArgs {
 
 __global__ __launch_bounds__(256) void k_reduce_compact(const uint8_t* __restrict__ flags,
                                                         const int32_t* __restrict__ counts, CompactArgs a,
-                                                        int16_t* __restrict__ idx, int32_t* __restrict__ binCount)
+                                                        int16_t* __restrict__ idx, int32_t* __restrict__ binCount,
+                                                        unsigned long long* hostSignal, uint32_t hostSeq)
 {
     __shared__ int waveSum[4];
     __shared__ int waveCnt[4];
@@ -1170,6 +1171,11 @@ __global__ __launch_bounds__(256) void k_reduce_compact(const uint8_t* __restric
             total = 1;
         }
         *binCount = total;
+        // Host-visible count without a copy: one 8-byte store (sequence number, count) into pinned host memory
+        // that the host polls; system scope, so it leaves the device at once.
+        if (hostSignal)
+            __hip_atomic_store(hostSignal, ((unsigned long long)hostSeq << 32) | (uint32_t)total, __ATOMIC_RELEASE,
+                               __HIP_MEMORY_SCOPE_SYSTEM);
     }
 }
 
@@ -1427,7 +1433,8 @@ size_t reduce_mask_workspace_bytes(int64_t totalBlocks)
 
 hipError_t launch_reduce_mask(const float* mask, const Geom& g, int bCntH, int bCntW, float tol,
                               bool avgPool, bool fixupZero, int16_t* activeBlockIndices,
-                              int32_t* binCountDevice, void* workspace, hipStream_t stream)
+                              int32_t* binCountDevice, void* workspace, hipStream_t stream,
+                              unsigned long long* hostSignal, uint32_t hostSeq)
 {
     const uint32_t T = (uint32_t)((int64_t)g.N * bCntH * bCntW);
     uint8_t* flags = static_cast<uint8_t*>(workspace);
@@ -1471,7 +1478,7 @@ hipError_t launch_reduce_mask(const float* mask, const Geom& g, int bCntH, int b
     c.fixupZero = fixupZero ? 1 : 0;
     c.dBw = p.dBw; c.dBhw = p.dBhw;
     hipLaunchKernelGGL(k_reduce_compact, dim3((T + 255) / 256), dim3(256), 0, stream, flags, counts, c,
-                       activeBlockIndices, binCountDevice);
+                       activeBlockIndices, binCountDevice, hostSignal, hostSeq);
     return hipGetLastError();
 }
 

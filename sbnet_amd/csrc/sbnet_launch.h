@@ -27,9 +27,13 @@ enum ScatterMode { SCATTER_ASSIGN = 0, SCATTER_ADD = 1, SCATTER_ATOMIC = 2 };
 // pooling workgroup, then one int32 for the total when the caller gives no device count.
 size_t reduce_mask_workspace_bytes(int64_t totalBlocks);
 
+// hostSignal (optional): device-visible address of an 8-byte word in pinned host memory; the kernel that knows
+// the count stores (hostSeq << 32 | count) there, so a host that polls the word needs no copy and no stream
+// synchronisation to learn the count.
 hipError_t launch_reduce_mask(const float* mask, const Geom& g, int bCntH, int bCntW, float tol,
                               bool avgPool, bool fixupZero, int16_t* activeBlockIndices,
-                              int32_t* binCountDevice, void* workspace, hipStream_t stream);
+                              int32_t* binCountDevice, void* workspace, hipStream_t stream,
+                              unsigned long long* hostSignal = nullptr, uint32_t hostSeq = 0);
 
 hipError_t launch_gather(const float* x, float* y, const int16_t* idx, int numActive,
                          const Geom& g, bool transpose, hipStream_t stream);

@@ -421,6 +421,63 @@ def test_image_of_2_pow_30_floats_takes_the_64_bit_offset_kernels():
     torch.cuda.empty_cache()
 
 
+def test_host_visible_count_is_never_stale_and_threads_do_not_mix():
+    """The host-visible count arrives through a polled word of pinned memory, one per thread: many calls in a row
+    with alternating masks must each report their own count, and two threads on two streams must not see each
+    other's; a call under stream capture must fail instead of waiting for a kernel that does not run."""
+    import threading
+    rng = np.random.default_rng(77)
+    H, W = 96, 96
+    bs, bst, bo = (8, 8), (8, 8), (0, 0)
+    bc = [12, 12]
+    masks = [(rng.random((1, H, W, 1)) < p).astype(np.float32) for p in (0.0005, 0.002, 0.01, 0.0)]
+    want = [int(orc.reduce_mask(m, bc, bs, bst, bo, 0.5, False)[1][0]) for m in masks]
+    assert len(set(want)) == len(want)
+    md = [dev(m) for m in masks]
+    for i in range(200):
+        r = sbnet_amd.reduce_mask(md[i % 4], bc, bs, bst, bo, tol=0.5)
+        assert int(r.bin_counts[0]) == want[i % 4]
+
+    errors = []
+
+    def worker(first):
+        try:
+            with torch.cuda.stream(torch.cuda.Stream()):
+                for i in range(150):
+                    k = (first + i) % 4
+                    r = sbnet_amd.reduce_mask(md[k], bc, bs, bst, bo, tol=0.5)
+                    if int(r.bin_counts[0]) != want[k]:
+                        errors.append((first, i, int(r.bin_counts[0]), want[k]))
+                        return
+        except Exception as e:  # noqa: BLE001
+            errors.append(repr(e))
+
+    threads = [threading.Thread(target=worker, args=(f,)) for f in (0, 1, 2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        sbnet_amd.reduce_mask(md[0], bc, bs, bst, bo, tol=0.5, sync=False)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    failed = False
+    with torch.cuda.graph(graph):
+        try:
+            sbnet_amd.reduce_mask(md[0], bc, bs, bst, bo, tol=0.5)  # host count: not possible while capturing
+        except RuntimeError:
+            failed = True
+        sbnet_amd.reduce_mask(md[0], bc, bs, bst, bo, tol=0.5, sync=False)
+    assert failed
+    torch.cuda.synchronize()
+
+
 def test_reduce_mask_rows_past_count_untouched():
     mask = np.zeros((1, 8, 8, 1), np.float32)
     mask[0, 0, 0, 0] = 1.0
