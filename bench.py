@@ -112,7 +112,7 @@ class Path:
                 s["idx"] = torch.from_numpy(idx_host).to(dev)
             s["ws"] = torch.empty(max(self.nws, 16), dtype=torch.uint8, device=dev)
             nsw = lib.sbnet_sparse_scatter_workspace_bytes(self.M, self.dims, 4, self.sbs, 2, self.sbst, 2, self.sbo, 2) \
-                if (wl.s_add and wl.s_atomic and not wl.transpose) else 0
+                if ((wl.s_add and wl.s_atomic and not wl.transpose) or not wl.s_var) else 0
             s["sws"] = torch.empty(nsw, dtype=torch.uint8, device=dev) if nsw else None
             s["dcount"] = torch.zeros(1, dtype=torch.int32, device=dev)
             if wl.x is not None:
@@ -400,6 +400,9 @@ def main():
                 "frac": round(g["GBps"] / HBM_PEAK_GBS, 4), "us_per_launch": g["us"],
                 "algorithmic_bytes_per_launch": g["bytes"],
                 "traffic": read_measured_traffic("gather_lines_scatter_planar_C3_30pct_pmc.txt")}
+    if roofline["traffic"]:
+        # the same launch time against the bytes the profiler counted between L2 and the fabric
+        roofline["traffic_GBps"] = round(roofline["traffic"] / g["us"] * 1e-3, 1)
     out = {
         "metric": "achieved HBM GB/s over reduce_mask+sparse_gather+sparse_scatter_var (algorithmic bytes / wall time per step); us/op and % of HBM peak under ops and roofline",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

@@ -156,8 +156,9 @@ int sbnet_sparse_gather_functor(const float* x, int N, int H, int W, int C, floa
  * sparse_scatter / sparse_scatter_var
  * ---------------------------------------------------------------------------------------- */
 
-/* Bytes of scratch that let an overlapping atomic scatter-add run without atomics (see workspace below);
-   0 when the method does not apply to this geometry. */
+/* Bytes of scratch that let an overlapping atomic scatter-add run without atomics and that let sparse_scatter
+   build its output in one pass instead of copying ybase first (see workspace below); 0 when neither applies to
+   this geometry. */
 size_t sbnet_sparse_scatter_workspace_bytes(int32_t num_active, const int64_t* ybase_dims, int ybase_rank,
                                             const int32_t* bsize, int bsize_len,
                                             const int32_t* bstride, int bstride_len,
@@ -178,7 +179,13 @@ size_t sbnet_sparse_scatter_workspace_bytes(int32_t num_active, const int64_t* y
  *   add=0 with overlapping blocks: as in the reference's GPU path, which block wins on an
  *   overlapped pixel is unspecified unless the overlapping values are equal.
  *   workspace   optional device scratch (4-byte aligned) of sbnet_sparse_scatter_workspace_bytes() bytes,
- *               or NULL.  It only matters for add=1, atomic=1; with it the overlapping adds need no atomics:
+ *               or NULL.  Two uses.
+ *               (1) sbnet_sparse_scatter with atomic=0: when the blocks cover 16 MB or more, y is built from
+ *               two disjoint parts instead of "copy ybase, scatter on top": pixels that no active block covers
+ *               are copied from ybase, covered ones are written by the scatter, which reads ybase where it
+ *               adds.  Same y, every byte moved once (one flag byte per pixel in the scratch tells the parts
+ *               apart).
+ *               (2) add=1, atomic=1: with it the overlapping adds need no atomics:
  *               - transpose=0 and at most 2x2 blocks per pixel: each pixel is summed by one owner in ascending
  *                 block-list order, bit-identical to the reference's sequential CPU functor;
  *               - otherwise (transpose=1, or up to 16 blocks per pixel): ceil(R/U)*ceil(S/V) passes of plain

@@ -347,7 +347,9 @@ size_t sbnet_sparse_scatter_workspace_bytes(int32_t num_active, const int64_t* y
                                     bsize, bstride, boffset);
     const size_t pull = sbnet::scatter_pull_workspace_bytes(g, num_active);
     const size_t color = sbnet::scatter_color_workspace_bytes(g, num_active);
-    return pull > color ? pull : color;
+    const size_t cover = sbnet::scatter_cover_workspace_bytes(g, num_active);
+    const size_t m = pull > color ? pull : color;
+    return m > cover ? m : cover;
 }
 
 static int scatter_op(const float* x, int32_t num_active, const int32_t* bin_counts_device,
@@ -371,6 +373,18 @@ static int scatter_op(const float* x, int32_t num_active, const int32_t* bin_cou
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (!geom_ok((int)ybase_dims[0], (int)ybase_dims[1], (int)ybase_dims[2], (int)ybase_dims[3], bsize, bstride))
         return SBNET_EINVAL_ARG;
+    // With scratch for one flag byte per pixel the output is built in one pass over its bytes: uncovered pixels
+    // are copied, covered ones written by the scatter (which reads ybase where it adds).
+    if (num_active > 0 && x && active_block_indices && !(add && atomic)) {
+        sbnet::Geom g = make_geom((int)ybase_dims[0], (int)ybase_dims[1], (int)ybase_dims[2], (int)ybase_dims[3], bsize,
+                                  bstride, boffset);
+        g.countDev = bin_counts_device;
+        bool done = false;
+        SBNET_HIP(sbnet::launch_scatter_over_base(x, ybase, y, active_block_indices, num_active, g, transpose != 0,
+                                                  add ? sbnet::SCATTER_ADD : sbnet::SCATTER_ASSIGN, workspace,
+                                                  workspace_bytes, s, done));
+        if (done) return SBNET_OK;
+    }
     SBNET_HIP(sbnet::launch_copy(y, ybase, count, s));  // sparse_gather.cc:338-346, no stream sync
     return scatter_impl(x, num_active, bin_counts_device, active_block_indices, y, ybase_dims, bsize, bstride, boffset,
                         add, atomic, transpose, workspace, workspace_bytes, s);

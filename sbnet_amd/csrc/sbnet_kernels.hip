@@ -260,7 +260,7 @@ __global__ __launch_bounds__(256) void k_gather_nhwc_wide(const float* __restric
 
 // sparse_gather.cc:103-130 with transpose == false.
 template <int VEC, int MODE>
-__global__ __launch_bounds__(256) void k_scatter_nhwc_wide(const float* __restrict__ x, float* __restrict__ y,
+__global__ __launch_bounds__(256) void k_scatter_nhwc_wide(const float* __restrict__ x, float* y, const float* ysrc,
                                                       const int16_t* __restrict__ idx, NhwcArgs a, ColorArgs col)
 {
     typedef typename Vec<VEC>::type vec;
@@ -279,7 +279,8 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc_wide(const float* __restri
     const int slo = max(0, -o.w0), shi = min(a.g.S, a.g.W - o.w0);
     const int lo = slo * CV, hi = shi * CV;
     const vec* __restrict__ xb = reinterpret_cast<const vec*>(x) + (size_t)ib * a.blockV;
-    vec* __restrict__ yv = reinterpret_cast<vec*>(y);
+    vec* yv = reinterpret_cast<vec*>(y);
+    const vec* ysv = reinterpret_cast<const vec*>(ysrc);  // what an add reads: y itself, or the base y is a copy of
     const uint32_t e0 = chunk * NHWC_CHUNK + lane;
 
     vec v[NHWC_UNR];
@@ -303,7 +304,7 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc_wide(const float* __restri
         vec cur[NHWC_UNR];
 #pragma unroll
         for (int u = 0; u < NHWC_UNR; ++u)
-            if (dst[u] >= 0) cur[u] = ld_stream(yv + dst[u]);
+            if (dst[u] >= 0) cur[u] = ld_stream(ysv + dst[u]);
 #pragma unroll
         for (int u = 0; u < NHWC_UNR; ++u)
             if (dst[u] >= 0) st_stream(yv + dst[u], vadd(cur[u], v[u]));
@@ -500,7 +501,7 @@ __global__ __launch_bounds__(256) void k_gather_nhwc(const float* __restrict__ x
 }
 
 template <int VEC, int MODE>
-__global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ x, float* __restrict__ y,
+__global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ x, float* y, const float* ysrc,
                                                       const int16_t* __restrict__ idx, NhwcArgs a, ColorArgs col)
 {
     typedef typename Vec<VEC>::type vec;
@@ -519,8 +520,9 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
     const int slo = max(0, -o.w0), shi = min(a.g.S, a.g.W - o.w0);
     const int lo = slo * CV, hi = shi * CV;
     const int64_t imgFloats = (int64_t)a.g.H * a.g.W * a.g.C;
-    float* __restrict__ img = y + (int64_t)o.n * imgFloats;
+    float* img = y + (int64_t)o.n * imgFloats;
     const rsrc_t yr = make_rsrc(img, (uint32_t)imgFloats * 4u);
+    const rsrc_t sr = make_rsrc(ysrc + (int64_t)o.n * imgFloats, (uint32_t)imgFloats * 4u);  // what an add reads
     const rsrc_t xr = make_rsrc(x + (int64_t)ib * a.blockV * VEC, a.blockV * (uint32_t)(VEC * 4));
     const uint32_t e0 = chunk * NHWC_CHUNK + lane;
     vec v[NHWC_UNR];
@@ -542,7 +544,7 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
     } else if (MODE == SCATTER_ADD || (MODE == SCATTER_COLOR && !atomics)) {
         vec cur[NHWC_UNR];
 #pragma unroll
-        for (int u = 0; u < NHWC_UNR; ++u) cur[u] = buf_load<VEC>(yr, dst[u]);
+        for (int u = 0; u < NHWC_UNR; ++u) cur[u] = buf_load<VEC>(sr, dst[u]);
 #pragma unroll
         for (int u = 0; u < NHWC_UNR; ++u) buf_store<BUF_NT>(yr, dst[u], vadd(cur[u], v[u]));
     } else {
@@ -845,7 +847,7 @@ __global__ __launch_bounds__(512) void k_gather_lines(const float* __restrict__ 
 
 // sparse_gather.cc:103-130 with transpose == true: the block stack is [blocks, C, R, S].
 template <int VEC, int MODE>
-__global__ __launch_bounds__(512) void k_scatter_planar(const float* __restrict__ x, float* __restrict__ y,
+__global__ __launch_bounds__(512) void k_scatter_planar(const float* __restrict__ x, float* y, const float* ysrc,
                                                         const int16_t* __restrict__ idx, TileArgs a, ColorArgs col)
 {
     typedef typename Vec<VEC>::type vec;
@@ -895,8 +897,9 @@ __global__ __launch_bounds__(512) void k_scatter_planar(const float* __restrict_
     // NHWC side: LDS -> base tensor; pixels outside the image are dropped (sparse_gather.cc:121)
     const BlockOrigin o = origin_of(raw, a.g);
     if (!o.valid) return;
-    float* __restrict__ img = y + (int64_t)o.n * a.imgFloats;
+    float* img = y + (int64_t)o.n * a.imgFloats;
     const rsrc_t yr = make_rsrc(img, a.imgBytes);
+    const rsrc_t sr = make_rsrc(ysrc + (int64_t)o.n * a.imgFloats, a.imgBytes);  // what an add reads
     const uint32_t c0l = (tid & ((1u << a.lppLog) - 1u)) * VEC;
     vec w[TILE_LD];
     uint32_t offs[TILE_LD];
@@ -917,7 +920,7 @@ __global__ __launch_bounds__(512) void k_scatter_planar(const float* __restrict_
     } else if (MODE == SCATTER_ADD || (MODE == SCATTER_COLOR && !atomics)) {
         vec cur[TILE_LD];
 #pragma unroll
-        for (int u = 0; u < TILE_LD; ++u) cur[u] = buf_load<VEC>(yr, offs[u]);
+        for (int u = 0; u < TILE_LD; ++u) cur[u] = buf_load<VEC>(sr, offs[u]);
 #pragma unroll
         for (int u = 0; u < TILE_LD; ++u) buf_store<BUF_NT>(yr, offs[u], vadd(cur[u], w[u]));
     } else {
@@ -936,7 +939,7 @@ __global__ __launch_bounds__(512) void k_scatter_planar(const float* __restrict_
 // not fit into a planar run: one thread per stack element.  The channel index varies fastest across
 // threads, so the NHWC side stays coalesced.
 template <int MODE, bool GATHER>
-__global__ __launch_bounds__(256) void k_planar_small(const float* __restrict__ x, float* __restrict__ y,
+__global__ __launch_bounds__(256) void k_planar_small(const float* __restrict__ x, float* y, const float* ysrc,
                                                       const int16_t* __restrict__ idx, Geom g, int64_t total)
 {
     const int RS = g.R * g.S;
@@ -955,7 +958,7 @@ __global__ __launch_bounds__(256) void k_planar_small(const float* __restrict__ 
             y[st] = in ? x[pix] : 0.f;
         } else if (in) {
             if (MODE == SCATTER_ASSIGN) y[pix] = x[st];
-            else if (MODE == SCATTER_ADD) y[pix] += x[st];
+            else if (MODE == SCATTER_ADD) y[pix] = ysrc[pix] + x[st];
             else atomic_add_f32(y + pix, x[st]);
         }
     }
@@ -1664,7 +1667,7 @@ static void gather_dispatch(const float* x, float* y, const int16_t* idx, const 
             const int64_t total = (int64_t)numActive * g.C * g.R * g.S;
             const int64_t wgs = (total + 255) / 256;
             hipLaunchKernelGGL((k_planar_small<SCATTER_ASSIGN, true>), dim3((unsigned)(wgs > 65536 ? 65536 : wgs)),
-                               dim3(256), 0, stream, x, y, idx, g, total);
+                               dim3(256), 0, stream, x, y, (const float*)y, idx, g, total);
             return;
         }
         hipLaunchKernelGGL(k_gather_planar<VEC>, tile_grid(a.grid2d, a.tpb, numActive, a.total), dim3(threads), lds,
@@ -1686,19 +1689,21 @@ hipError_t launch_gather(const float* x, float* y, const int16_t* idx, int numAc
     return hipGetLastError();
 }
 
+// `ysrc` is what an add reads: y itself for the in-place op, the base tensor when y is being built as
+// "copy of the base + scatter" without copying the covered pixels first.
 template <int VEC, int MODE>
-static void scatter_dispatch(const float* x, float* y, const int16_t* idx, const Geom& g, int numActive,
-                             bool transpose, hipStream_t stream, hipError_t& err)
+static void scatter_dispatch(const float* x, float* y, const float* ysrc, const int16_t* idx, const Geom& g,
+                             int numActive, bool transpose, hipStream_t stream, hipError_t& err)
 {
     if (!transpose) {
         NhwcArgs a;
         if (!make_nhwc_args(g, numActive, VEC, a)) { err = hipErrorInvalidValue; return; }
         if (nhwc_fits_buffers(g))
-            hipLaunchKernelGGL((k_scatter_nhwc<VEC, MODE>), dim3((a.units + 3) / 4), dim3(256), 0, stream, x, y, idx,
-                               a, ColorArgs{1, 1, 0, nullptr});
+            hipLaunchKernelGGL((k_scatter_nhwc<VEC, MODE>), dim3((a.units + 3) / 4), dim3(256), 0, stream, x, y, ysrc,
+                               idx, a, ColorArgs{1, 1, 0, nullptr});
         else
             hipLaunchKernelGGL((k_scatter_nhwc_wide<VEC, MODE>), dim3((a.units + 3) / 4), dim3(256), 0, stream, x, y,
-                               idx, a, ColorArgs{1, 1, 0, nullptr});
+                               ysrc, idx, a, ColorArgs{1, 1, 0, nullptr});
     } else {
         TileArgs a;
         int threads;
@@ -1709,34 +1714,45 @@ static void scatter_dispatch(const float* x, float* y, const int16_t* idx, const
             const int64_t total = (int64_t)numActive * g.C * g.R * g.S;
             const int64_t wgs = (total + 255) / 256;
             hipLaunchKernelGGL((k_planar_small<MODE, false>), dim3((unsigned)(wgs > 65536 ? 65536 : wgs)), dim3(256),
-                               0, stream, x, y, idx, g, total);
+                               0, stream, x, y, ysrc, idx, g, total);
             return;
         }
         hipLaunchKernelGGL((k_scatter_planar<VEC, MODE>), tile_grid(a.grid2d, a.tpb, numActive, a.total), dim3(threads),
-                           lds, stream, x, y, idx, a, ColorArgs{1, 1, 0, nullptr});
+                           lds, stream, x, y, ysrc, idx, a, ColorArgs{1, 1, 0, nullptr});
     }
 }
 
 template <int VEC>
-static void scatter_mode(const float* x, float* y, const int16_t* idx, const Geom& g, int numActive,
+static void scatter_mode(const float* x, float* y, const float* ysrc, const int16_t* idx, const Geom& g, int numActive,
                          bool transpose, ScatterMode mode, hipStream_t stream, hipError_t& err)
 {
-    if (mode == SCATTER_ASSIGN) scatter_dispatch<VEC, SCATTER_ASSIGN>(x, y, idx, g, numActive, transpose, stream, err);
-    else if (mode == SCATTER_ADD) scatter_dispatch<VEC, SCATTER_ADD>(x, y, idx, g, numActive, transpose, stream, err);
-    else scatter_dispatch<VEC, SCATTER_ATOMIC>(x, y, idx, g, numActive, transpose, stream, err);
+    if (mode == SCATTER_ASSIGN)
+        scatter_dispatch<VEC, SCATTER_ASSIGN>(x, y, ysrc, idx, g, numActive, transpose, stream, err);
+    else if (mode == SCATTER_ADD)
+        scatter_dispatch<VEC, SCATTER_ADD>(x, y, ysrc, idx, g, numActive, transpose, stream, err);
+    else
+        scatter_dispatch<VEC, SCATTER_ATOMIC>(x, y, ysrc, idx, g, numActive, transpose, stream, err);
+}
+
+static hipError_t scatter_from(const float* x, float* y, const float* ysrc, const int16_t* idx, int numActive,
+                               const Geom& g, bool transpose, ScatterMode mode, hipStream_t stream)
+{
+    if (numActive == 0) return hipSuccess;
+    hipError_t err = hipSuccess;
+    int vec = pick_vec(g, y, transpose ? nullptr : x);
+    const int vsrc = pick_vec(g, ysrc, nullptr);
+    if (vsrc < vec) vec = vsrc;
+    if (vec == 4) scatter_mode<4>(x, y, ysrc, idx, g, numActive, transpose, mode, stream, err);
+    else if (vec == 2) scatter_mode<2>(x, y, ysrc, idx, g, numActive, transpose, mode, stream, err);
+    else scatter_mode<1>(x, y, ysrc, idx, g, numActive, transpose, mode, stream, err);
+    if (err != hipSuccess) return err;
+    return hipGetLastError();
 }
 
 hipError_t launch_scatter(const float* x, float* y, const int16_t* idx, int numActive, const Geom& g,
                           bool transpose, ScatterMode mode, hipStream_t stream)
 {
-    if (numActive == 0) return hipSuccess;
-    hipError_t err = hipSuccess;
-    const int vec = pick_vec(g, y, transpose ? nullptr : x);
-    if (vec == 4) scatter_mode<4>(x, y, idx, g, numActive, transpose, mode, stream, err);
-    else if (vec == 2) scatter_mode<2>(x, y, idx, g, numActive, transpose, mode, stream, err);
-    else scatter_mode<1>(x, y, idx, g, numActive, transpose, mode, stream, err);
-    if (err != hipSuccess) return err;
-    return hipGetLastError();
+    return scatter_from(x, y, y, idx, numActive, g, transpose, mode, stream);
 }
 
 // Extent of the inverse block map (blocks that can touch the image); false when it cannot be built.
@@ -1843,10 +1859,10 @@ static bool color_passes(const float* x, float* y, const int16_t* idx, const Geo
         for (col.pass = 0; col.pass < passes; ++col.pass) {
             if (buf)
                 hipLaunchKernelGGL((k_scatter_nhwc<VEC, SCATTER_COLOR>), dim3((a.units + 3) / 4), dim3(256), 0, stream,
-                                   x, y, idx, a, col);
+                                   x, y, (const float*)y, idx, a, col);
             else
                 hipLaunchKernelGGL((k_scatter_nhwc_wide<VEC, SCATTER_COLOR>), dim3((a.units + 3) / 4), dim3(256), 0,
-                                   stream, x, y, idx, a, col);
+                                   stream, x, y, (const float*)y, idx, a, col);
         }
     } else {
         TileArgs a;
@@ -1856,7 +1872,7 @@ static bool color_passes(const float* x, float* y, const int16_t* idx, const Geo
         if ((int64_t)g.R * g.S < 4 || !make_tile_args(g, numActive, VEC, a, threads, lds, grid, 16 * 1024)) return false;
         for (col.pass = 0; col.pass < passes; ++col.pass)
             hipLaunchKernelGGL((k_scatter_planar<VEC, SCATTER_COLOR>), tile_grid(a.grid2d, a.tpb, numActive, a.total),
-                               dim3(threads), lds, stream, x, y, idx, a, col);
+                               dim3(threads), lds, stream, x, y, (const float*)y, idx, a, col);
     }
     return true;
 }
@@ -1904,6 +1920,126 @@ hipError_t launch_scatter_colored(const float* x, float* y, const int16_t* idx, 
     else color_passes<1>(x, y, idx, g, numActive, transpose, col, passes, stream);
     done = true;
     return hipGetLastError();
+}
+
+// ---- "copy of the base + scatter" without copying what the scatter overwrites -------------------
+//
+// sparse_scatter (not the in-place op) returns a fresh tensor: the base, with the blocks written or added on
+// top (sparse_gather.cc:338-346 copies the whole base, then scatters).  Copy-then-scatter moves every
+// covered pixel twice more than needed.  With one flag byte per pixel ("an active block covers it") the work
+// splits into two disjoint parts: k_copy_uncovered copies the pixels without the flag, and the ordinary
+// scatter kernels write the flagged ones, reading the base (`ysrc`) where they add.  Same result, every byte
+// moved once.  The flags cost N*H*W bytes of scratch and two small launches (clear, mark).
+
+struct CoverArgs {
+    Geom g;
+    uint32_t RS;
+    uint32_t imgV;      // vectors per image
+    uint32_t imgBytes;
+    int64_t imgFloats, imgPixels;
+    FastDiv dCV, dS;
+};
+
+constexpr int COVER_UNR = 4;
+
+__global__ __launch_bounds__(256) void k_cover_clear(uint32_t* __restrict__ words, int64_t n)
+{
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) words[i] = 0u;
+}
+
+// One thread per (block, block pixel): flags the pixel if it lies inside the image.  Blocks past the device-
+// resident count and rows with an image number outside [0, N) flag nothing, as they scatter nothing.
+__global__ __launch_bounds__(256) void k_cover_mark(const int16_t* __restrict__ idx, int numActive, CoverArgs a,
+                                                    uint8_t* __restrict__ flags)
+{
+    const int64_t total = (int64_t)numActive * a.RS;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const uint32_t ib = (uint32_t)(i / a.RS);
+        if (a.g.countDev && ib >= (uint32_t)*a.g.countDev) return;
+        const uint32_t p = (uint32_t)(i - (int64_t)ib * a.RS);
+        const uint32_t r = fdiv(p, a.dS), sc = p - r * (uint32_t)a.g.S;
+        const BlockOrigin o = load_origin(idx, ib, a.g);
+        const int hh = o.h0 + (int)r, ww = o.w0 + (int)sc;
+        if (o.valid && (unsigned)hh < (unsigned)a.g.H && (unsigned)ww < (unsigned)a.g.W)
+            flags[(int64_t)o.n * a.imgPixels + (int64_t)hh * a.g.W + ww] = 1;
+    }
+}
+
+template <int VEC>
+__global__ __launch_bounds__(256) void k_copy_uncovered(const float* __restrict__ src, float* __restrict__ dst,
+                                                        const uint8_t* __restrict__ flags, CoverArgs a)
+{
+    typedef typename Vec<VEC>::type vec;
+    const uint32_t n = blockIdx.y;
+    const rsrc_t sr = make_rsrc(src + (int64_t)n * a.imgFloats, a.imgBytes);
+    const rsrc_t dr = make_rsrc(dst + (int64_t)n * a.imgFloats, a.imgBytes);
+    const uint8_t* __restrict__ fl = flags + (int64_t)n * a.imgPixels;
+    const uint32_t e0 = blockIdx.x * (256u * COVER_UNR) + threadIdx.x;
+    uint8_t cov[COVER_UNR];
+#pragma unroll
+    for (int u = 0; u < COVER_UNR; ++u) {
+        const uint32_t e = min(e0 + (uint32_t)u * 256u, a.imgV - 1u);
+        cov[u] = fl[fdiv(e, a.dCV)];
+    }
+    uint32_t off[COVER_UNR];
+#pragma unroll
+    for (int u = 0; u < COVER_UNR; ++u) {
+        const uint32_t e = e0 + (uint32_t)u * 256u;
+        off[u] = (e >= a.imgV || cov[u]) ? BUF_OOB : e * (uint32_t)(VEC * 4);
+    }
+    vec v[COVER_UNR];
+#pragma unroll
+    for (int u = 0; u < COVER_UNR; ++u) v[u] = buf_load<VEC>(sr, off[u]);
+#pragma unroll
+    for (int u = 0; u < COVER_UNR; ++u) buf_store<BUF_NT>(dr, off[u], v[u]);
+}
+
+size_t scatter_cover_workspace_bytes(const Geom& g, int numActive)
+{
+    if (numActive <= 0) return 0;
+    if ((int64_t)g.H * g.W * g.C >= (1ll << 30)) return 0;  // 32-bit byte offsets inside one image
+    if ((int64_t)g.R * g.S >= (1ll << 31)) return 0;
+    return (((size_t)g.N * g.H * g.W + 3) & ~(size_t)3) + 16;
+}
+
+hipError_t launch_scatter_over_base(const float* x, const float* ybase, float* y, const int16_t* idx, int numActive,
+                                    const Geom& g, bool transpose, ScatterMode mode, void* workspace,
+                                    size_t workspaceBytes, hipStream_t stream, bool& done)
+{
+    done = false;
+    if (mode == SCATTER_ATOMIC || numActive <= 0) return hipSuccess;
+    const size_t need = scatter_cover_workspace_bytes(g, numActive);
+    if (!workspace || need == 0 || workspaceBytes < need || (reinterpret_cast<uintptr_t>(workspace) & 3))
+        return hipSuccess;
+    // Two small launches prepare the flags: worth it once the blocks cover enough of the tensor to pay for them
+    // (each covered byte saves one read and one write of the copy).
+    if ((int64_t)numActive * g.R * g.S * g.C * 4 < (16ll << 20)) return hipSuccess;
+
+    CoverArgs c;
+    c.g = g;
+    c.RS = (uint32_t)(g.R * g.S);
+    const int vec = pick_vec(g, ybase, y);
+    c.imgFloats = (int64_t)g.H * g.W * g.C;
+    c.imgPixels = (int64_t)g.H * g.W;
+    c.imgV = (uint32_t)(c.imgFloats / vec);
+    c.imgBytes = (uint32_t)(c.imgFloats * 4);
+    c.dCV = make_fastdiv((uint32_t)(g.C / vec));
+    c.dS = make_fastdiv((uint32_t)g.S);
+    uint8_t* flags = static_cast<uint8_t*>(workspace);
+
+    const int64_t words = (int64_t)((need - 16) / 4);
+    int64_t wgs = (words + 255) / 256;
+    if (wgs > 8192) wgs = 8192;
+    hipLaunchKernelGGL(k_cover_clear, dim3((unsigned)wgs), dim3(256), 0, stream, reinterpret_cast<uint32_t*>(flags), words);
+    int64_t markWgs = ((int64_t)numActive * c.RS + 255) / 256;
+    if (markWgs > 65536) markWgs = 65536;
+    hipLaunchKernelGGL(k_cover_mark, dim3((unsigned)markWgs), dim3(256), 0, stream, idx, numActive, c, flags);
+    const dim3 grid((c.imgV + 256u * COVER_UNR - 1) / (256u * COVER_UNR), (unsigned)g.N);
+    if (vec == 4) hipLaunchKernelGGL(k_copy_uncovered<4>, grid, dim3(256), 0, stream, ybase, y, flags, c);
+    else if (vec == 2) hipLaunchKernelGGL(k_copy_uncovered<2>, grid, dim3(256), 0, stream, ybase, y, flags, c);
+    else hipLaunchKernelGGL(k_copy_uncovered<1>, grid, dim3(256), 0, stream, ybase, y, flags, c);
+    done = true;
+    return scatter_from(x, y, ybase, idx, numActive, g, transpose, mode, stream);
 }
 
 hipError_t launch_copy(float* dst, const float* src, size_t count, hipStream_t stream)

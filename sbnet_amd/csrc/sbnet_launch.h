@@ -56,6 +56,16 @@ hipError_t launch_scatter_colored(const float* x, float* y, const int16_t* idx, 
                                   bool transpose, void* workspace, size_t workspaceBytes, hipStream_t stream,
                                   bool& done);
 
+// y = copy of ybase with the blocks written ("=") or added ("+=", non-overlapping) on top, moving every byte once:
+// pixels that no active block covers are copied, covered ones are written by the scatter kernels, which read
+// ybase where they add.  Needs scratch of scatter_cover_workspace_bytes() for one flag byte per pixel; `done` is
+// false when the method does not apply (no scratch, atomic mode, too little coverage to pay for preparing the
+// flags) and nothing was launched: the caller then copies ybase and scatters in place.
+size_t scatter_cover_workspace_bytes(const Geom& g, int numActive);
+hipError_t launch_scatter_over_base(const float* x, const float* ybase, float* y, const int16_t* idx, int numActive,
+                                    const Geom& g, bool transpose, ScatterMode mode, void* workspace,
+                                    size_t workspaceBytes, hipStream_t stream, bool& done);
+
 hipError_t launch_copy(float* dst, const float* src, size_t count, hipStream_t stream);
 
 }  // namespace sbnet

@@ -194,8 +194,9 @@ def scatter_forward(x, bin_counts, active_block_indices, ybase, dynamic_bsize, d
     dims, rank = _dims(ybase)
     with torch.cuda.device(ybase.device):
         ws_ptr, ws_bytes = None, 0
-        if add and atomic:
-            # scratch for the atomic-free scatter-add of overlapping blocks
+        if (add and atomic) or not use_var:
+            # scratch for the atomic-free scatter-add of overlapping blocks, and for building the copying op's
+            # output in one pass (uncovered pixels copied, covered ones scattered)
             need = lib.sbnet_sparse_scatter_workspace_bytes(M, dims, rank, bsp, bsl, btp, btl, bop, bol)
             if need:
                 ws = _workspace(ybase.device, need)

@@ -53,14 +53,20 @@ def test_size_queries():
 def test_scatter_workspace_query():
     lib = _lib.load()
     dims = I64x4(2, 512, 512, 256)
+    flags = 2 * 512 * 512 + 16   # one flag byte per pixel: the copying scatter built in one pass
     # 16x16 blocks at stride 8: 2x2 blocks cover a pixel, the atomic-free method applies
     n = lib.sbnet_sparse_scatter_workspace_bytes(2000, dims, 4, I32x2(16, 16), 2, I32x2(8, 8), 2, I32x2(0, 0), 2)
-    assert n >= 2 * 64 * 64 * 4 + 2000 * 4
+    assert n >= max(2 * 64 * 64 * 4 + 2000 * 4, flags)
     # 16x16 at stride 4: 4x4 blocks cover a pixel: the add runs in 16 passes, which needs the block map only
+    # (less than the flag bytes here)
     n = lib.sbnet_sparse_scatter_workspace_bytes(2000, dims, 4, I32x2(16, 16), 2, I32x2(4, 4), 2, I32x2(0, 0), 2)
-    assert 2 * 128 * 128 * 4 <= n < 2 * 140 * 140 * 4
-    # 16x16 at stride 3: 6x6 blocks cover a pixel, beyond both methods
+    assert n == max(flags, n) and 2 * 128 * 128 * 4 <= n < max(2 * 140 * 140 * 4, flags + 1)
+    # 16x16 at stride 3: 6x6 blocks cover a pixel, beyond both atomic-free methods: the flag bytes only
     assert lib.sbnet_sparse_scatter_workspace_bytes(2000, dims, 4, I32x2(16, 16), 2, I32x2(3, 3), 2, I32x2(0, 0),
+                                                    2) == flags
+    # an image of 2^30 floats or more is beyond the one-pass copy as well
+    big = I64x4(1, 32768, 32768, 1)
+    assert lib.sbnet_sparse_scatter_workspace_bytes(2000, big, 4, I32x2(16, 16), 2, I32x2(3, 3), 2, I32x2(0, 0),
                                                     2) == 0
     assert lib.sbnet_sparse_scatter_workspace_bytes(2000, dims, 3, I32x2(16, 16), 2, I32x2(8, 8), 2, I32x2(0, 0),
                                                     2) == 0

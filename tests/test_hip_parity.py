@@ -478,6 +478,51 @@ def test_host_visible_count_is_never_stale_and_threads_do_not_mix():
     torch.cuda.synchronize()
 
 
+@pytest.mark.parametrize("geom", [
+    # (N, H, W, C), bsize, bstride, boffset, keep probability, add
+    ((2, 200, 200, 64), (16, 16), (16, 16), (0, 0), 0.9, True),
+    ((2, 200, 200, 64), (16, 16), (16, 16), (0, 0), 0.9, False),
+    ((2, 256, 256, 64), (18, 18), (16, 16), (-1, -1), 0.8, False),   # overlapping blocks
+    ((4, 256, 256, 64), (5, 7), (8, 9), (2, -3), 1.0, True),         # gaps, uneven offsets
+    ((1, 512, 512, 30), (9, 9), (9, 9), (-4, 3), 0.95, True),        # 8-byte vectors
+    ((1, 1200, 1100, 7), (11, 13), (11, 13), (0, 0), 1.0, True),     # 4-byte vectors
+    ((1, 800, 800, 32), (27, 27), (25, 25), (-1, -1), 0.9, False),   # plane split over several tiles
+], ids=lambda g: "x".join(map(str, g[0])) + "_b%dx%d" % g[1])
+def test_copying_scatter_moves_every_byte_once(geom):
+    """sparse_scatter (the op that returns a new tensor) with enough coverage builds its output from two disjoint
+    parts -- pixels no active block covers are copied from ybase, covered ones written by the scatter, which
+    reads ybase where it adds -- instead of copying ybase and scattering on top.  Same result, bit for bit, for
+    both stack layouts, with the count on the host and on the device; ybase is left alone."""
+    (N, H, W, C), bs, bst, bo, keep, add = geom
+    rng = np.random.default_rng(hash(geom[0]) % 1000)
+    bc = bcount_covering(H, W, bst, bo)
+    allb = np.array([(n, i, j) for n in range(N) for i in range(bc[0]) for j in range(bc[1])], np.int16)
+    idx = allb[rng.random(len(allb)) < keep]
+    cnt = np.array([len(idx)], np.int32)
+    assert len(idx) * bs[0] * bs[1] * C * 4 >= 16 << 20   # enough coverage for the one-pass path
+    x = rng.standard_normal((N, H, W, C)).astype(np.float32)
+    base = rng.standard_normal((N, H, W, C)).astype(np.float32)
+    idx_d, cnt_t, base_d = dev(idx), torch.from_numpy(cnt), dev(base)
+    cnt_d = cnt_t.to(DEV)
+    for transpose in (False, True):
+        stack = orc.sparse_gather(x, cnt, idx, bs, bst, bo, transpose=transpose)   # overlaps carry equal values
+        y_o = orc.sparse_scatter(stack, cnt, idx, base, bs, bst, bo, add=add, transpose=transpose)
+        stack_d = dev(stack)
+        y = sbnet_amd.sparse_scatter(stack_d, cnt_t, idx_d, base_d, bs, bst, bo, add=add, transpose=transpose)
+        assert y.data_ptr() != base_d.data_ptr()
+        np.testing.assert_array_equal(host(y), y_o)
+        y2 = sbnet_amd.sparse_scatter(stack_d, cnt_d, idx_d, base_d, bs, bst, bo, add=add, transpose=transpose)
+        np.testing.assert_array_equal(host(y2), y_o)
+        np.testing.assert_array_equal(host(base_d), base)
+    # a base that is only 4-byte aligned takes the narrow copies
+    flat = torch.empty(base_d.numel() + 1, device=DEV)
+    mis = flat[1:].view(base_d.shape)
+    mis.copy_(base_d)
+    y_o = orc.sparse_scatter(stack, cnt, idx, base, bs, bst, bo, add=add, transpose=True)
+    y3 = sbnet_amd.sparse_scatter(stack_d, cnt_t, idx_d, mis, bs, bst, bo, add=add, transpose=True)
+    np.testing.assert_array_equal(host(y3), y_o)
+
+
 def test_reduce_mask_rows_past_count_untouched():
     mask = np.zeros((1, 8, 8, 1), np.float32)
     mask[0, 0, 0, 0] = 1.0
