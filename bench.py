@@ -309,7 +309,7 @@ def main():
     args = parse()
     if args.gpus != 1:
         print("bench.py: this path is measured on one GPU only (one MI355X per box); --gpus %d is not supported. "
-              "Sharding is by image (n) with no exchange; see DESIGN.md." % args.gpus, file=sys.stderr)
+              "The path shards by image (n) with no exchange between GPUs." % args.gpus, file=sys.stderr)
         sys.exit(2)
     import torch
     if not torch.cuda.is_available():

@@ -72,7 +72,7 @@ REDUCE = [
 
 
 def config1_inputs(seed=1001):
-    """BASELINE config 1: x [1,64,64,16] ~U(-1,1); mask = 8x8 grid of 8x8 tiles, each 1 w.p. 0.5."""
+    """Benchmark configuration 1: x [1,64,64,16] ~U(-1,1); mask = 8x8 grid of 8x8 tiles, each 1 w.p. 0.5."""
     rng = np.random.default_rng(seed)
     x = rng.uniform(-1.0, 1.0, size=(1, 64, 64, 16)).astype(np.float32)
     tiles = (rng.random((8, 8)) < 0.5).astype(np.float32)
