@@ -94,10 +94,17 @@ class Path:
             idx_host = np.ascontiguousarray(wl.indices, np.int16)
             self.M = len(idx_host)
         else:
-            from oracle import sbnet_oracle as orc  # only to size the buffers (M); not timed, not the product path
-            idx_host, cnt = orc.reduce_mask(wl.mask, wl.bcount, wl.bsize, wl.bstride, wl.boffset, wl.tol, wl.avgpool)
-            self.M = int(cnt[0])
-            idx_host = idx_host[:self.M]
+            # the block list comes from the library's own reduce_mask (untimed): it sizes the buffers
+            mask_d = torch.from_numpy(wl.mask).to(dev)
+            idx_d = torch.zeros((self.maxidx, 3), dtype=torch.int16, device=dev)
+            ws_d = torch.empty(max(self.nws, 16), dtype=torch.uint8, device=dev)
+            self.check(lib.sbnet_reduce_mask(mask_d.data_ptr(), N, H, W, self.bc, 2, self.bs, 2, self.bst, 2, self.bo, 2,
+                                             wl.tol, int(wl.avgpool), idx_d.data_ptr(), self.hc_ptr, None,
+                                             ws_d.data_ptr(), self.nws, self.stream))
+            torch.cuda.synchronize()
+            self.M = int(self.host_count[0])
+            idx_host = idx_d[:self.M].cpu().numpy()
+            del mask_d, idx_d, ws_d
         self.idx_host = idx_host
         R, S = wl.bsize
         sR, sS = wl.s_bsize
