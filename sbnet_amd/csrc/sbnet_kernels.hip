@@ -680,9 +680,10 @@ __global__ __launch_bounds__(512) void k_gather_planar(const float* __restrict__
 // plane is split over several tiles; a tile of whole planes already writes one contiguous piece.
 //
 // LDS: row c at c*Pp, window pixel q at column q + phi(c), phi(c) = (c*RS + p0) & 3, XOR-swizzled as
-// above.  The shift phi makes LDS columns congruent to l modulo 4, so an output slot that lies inside
-// one row is one ds_read_b128.  Slots that cross into the next row (up to 9 per row, and only in the
-// last split) are assembled from four 4-byte reads.
+// above.  The shift phi makes LDS columns congruent to l modulo 4, so every output slot is one
+// ds_read_b128.  In the last split the wrapped pixels of channel c (the first pixels of its plane) are
+// stored behind the pixels of channel c-1 instead, where l continues: the slots of row c-1's last line
+// that cross into plane c are then contiguous in LDS like any other.
 
 constexpr int LINE_FLOATS = 32;
 constexpr int LINE_EXT = LINE_FLOATS - 1;
@@ -760,9 +761,14 @@ __global__ __launch_bounds__(512) void k_gather_lines(const float* __restrict__ 
         }
         if (r >= (uint32_t)a.g.R) r -= (uint32_t)a.g.R;
     }
-    // registers -> LDS.  With a pixel step that is a multiple of 32 the swizzle (bits 2..4 of the column) does
-    // not depend on u, and the column of (u, k) is the column of (0, k) plus u*step.
-    {
+    // registers -> LDS.  In the last split of a plane the window wraps: its pixels from `wrapStart` on are the
+    // first pixels of the plane, which the output needs as the continuation of the PREVIOUS channel's row (the
+    // last line of row c-1 runs into row c).  They are stored there, behind row c-1's own pixels, so that every
+    // output slot is one aligned 16-byte LDS read; channel 0 of the chunk has no predecessor and drops them.
+    const uint32_t wrapStart = (p1 == RS && p0 != 0u) ? RS - p0 : 0xFFFFFFFFu;
+    if (wrapStart == 0xFFFFFFFFu) {
+        // With a pixel step that is a multiple of 32 the swizzle (bits 2..4 of the column) does not depend on u,
+        // and the column of (u, k) is the column of (0, k) plus u*step.
         const uint32_t swz = lds_swz(cl * 4u);
         uint32_t rowAddr[4];
 #pragma unroll
@@ -791,6 +797,42 @@ __global__ __launch_bounds__(512) void k_gather_lines(const float* __restrict__ 
                 }
             }
         }
+    } else if ((step & 31u) == 0) {
+        // the same with the wrapped pixels one row up: rows 4*cl+k-1 are this thread's own rows 4*cl+k-1 for
+        // k >= 1 (same swizzle group), and row 4*cl-1 for k = 0
+        const uint32_t swz = lds_swz(cl * 4u);
+        uint32_t rowAddr[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t phi = ((uint32_t)k * RS + p0) & 3u;
+            rowAddr[k] = (cl * 4u + (uint32_t)k) * (uint32_t)a.Pp + ((phi + q0) ^ swz);
+        }
+        const uint32_t rowP = cl * 4u - 1u;  // no such row for cl == 0: channel 0 drops its wrapped pixels
+        const uint32_t addrP = rowP * (uint32_t)a.Pp + ((((rowP * RS + p0) & 3u) + q0) ^ lds_swz(rowP));
+#pragma unroll
+        for (int u = 0; u < LD; ++u) {
+            const uint32_t q = q0 + (uint32_t)u * step;
+            if (q < win) {
+                const bool wr = q >= wrapStart;
+                if (!(wr && cl == 0u)) lds[(wr ? addrP : rowAddr[0]) + (uint32_t)u * step] = vget(v[u], 0);
+#pragma unroll
+                for (int k = 1; k < 4; ++k) lds[(wr ? rowAddr[k - 1] : rowAddr[k]) + (uint32_t)u * step] = vget(v[u], k);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int u = 0; u < LD; ++u) {
+            const uint32_t q = q0 + (uint32_t)u * step;
+            if (q < win) {
+                const uint32_t back = q >= wrapStart ? 1u : 0u;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t row = cl * 4u + (uint32_t)k - back;  // 0xFFFFFFFF for channel 0's wrapped pixels
+                    const uint32_t phi = (row * RS + p0) & 3u;
+                    if (row != 0xFFFFFFFFu) lds[row * (uint32_t)a.Pp + ((phi + q) ^ lds_swz(row))] = vget(v[u], k);
+                }
+            }
+        }
     }
     lds_barrier();
 
@@ -801,7 +843,7 @@ __global__ __launch_bounds__(512) void k_gather_lines(const float* __restrict__ 
     const rsrc_t yr = make_rsrc(y + chunkBase, chunkFloats * 4u);
     {
         // One wave per row, four rows in flight: everything about the row (its range [A, B) of whole lines,
-        // where it ends, its swizzle) is wave-uniform and stays on the scalar unit; a lane only adds 4*k.
+        // its swizzle) is wave-uniform and stays on the scalar unit; a lane only adds 4*k.
         const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
         const uint32_t lane = tid & 63u, nwaves = nthr >> 6;
         for (uint32_t cr0 = wave; cr0 < ctEff; cr0 += 4u * nwaves) {
@@ -816,26 +858,12 @@ __global__ __launch_bounds__(512) void k_gather_lines(const float* __restrict__ 
                     const uint32_t B = (cr >= ctEff)          ? 0u
                                        : (lin1 == chunkFloats) ? chunkFloats
                                                                : ((a0 + lin1 + LINE_EXT) & ~(uint32_t)LINE_EXT) - a0;
-                    const uint32_t rowEnd = lin0 - p0 + RS;
                     const uint32_t colBase = A - lin0 + (lin0 & 3u);  // multiple of 4 less than 36
                     const uint32_t k4 = 4u * (kb + lane);
                     const uint32_t l = A + k4;
                     const bool live = l < B;
-                    const bool inrow = l + 4u <= rowEnd;
-                    qv[u] = lds_read4(lds + ((live && inrow) ? cr * (uint32_t)a.Pp + ((colBase + k4) ^ lds_swz(cr)) : 0u));
-                    if (live && !inrow) {
-                        // only in the last split: the row's last line runs into the first pixels of the next plane,
-                        // which sit at the end of the cyclic window
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            const uint32_t le = l + (uint32_t)e;
-                            const uint32_t ce = le >= rowEnd ? cr + 1u : cr;  // RS > LINE_EXT here: one crossing at most
-                            const uint32_t pe = le - ce * RS;
-                            const uint32_t qe = pe < p0 ? pe + RS - p0 : pe - p0;
-                            const uint32_t phi = (ce * RS + p0) & 3u;
-                            vset(qv[u], e, lds[ce * (uint32_t)a.Pp + ((qe + phi) ^ lds_swz(ce))]);
-                        }
-                    }
+                    // (a row's last line may run into the next plane: those pixels sit behind the row in LDS)
+                    qv[u] = lds_read4(lds + (live ? cr * (uint32_t)a.Pp + ((colBase + k4) ^ lds_swz(cr)) : 0u));
                     off[u] = live ? l * 4u : BUF_OOB;
                 }
 #pragma unroll
