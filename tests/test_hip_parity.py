@@ -523,6 +523,46 @@ def test_copying_scatter_moves_every_byte_once(geom):
     np.testing.assert_array_equal(host(y3), y_o)
 
 
+@pytest.mark.parametrize("case", [
+    # (H, W, C), bsize, bstride, boffset, block list (n, bh, bw)
+    ((20, 30, 8), (6, 7), (6, 7), (0, 0), []),                                   # empty list
+    ((20, 30, 8), (6, 7), (6, 7), (0, 0), [(0, 50, 0), (0, 0, 90), (0, -9, -9)]),  # blocks wholly outside the image
+    ((20, 30, 8), (6, 7), (6, 7), (-40, -40), [(0, 0, 0), (0, 6, 5), (0, 7, 6)]),  # far negative offsets
+    ((5, 4, 12), (9, 11), (9, 11), (-2, -3), [(0, 0, 0)]),                       # a block larger than the image
+    ((1, 37, 4), (1, 5), (1, 5), (0, -1), [(0, 0, 0), (0, 0, 3), (0, 0, 7)]),      # one-row image
+    ((41, 1, 6), (4, 1), (4, 1), (-1, 0), [(0, 0, 0), (0, 5, 0), (0, 10, 0)]),     # one-column image
+    ((16, 16, 3), (4, 4), (4, 4), (0, 0), [(1, 3, 3), (0, 0, 0), (1, 0, 0), (0, 3, 3)]),  # list not in order, N = 2
+], ids=["empty", "outside", "far_offset", "block_gt_image", "one_row", "one_column", "unordered"])
+def test_edge_geometries(case):
+    """Lists and geometries at the edges of what the ops accept: nothing to do, blocks that miss the image
+    (gather pads with zeros, scatter drops), blocks larger than the image, degenerate images, an arbitrary
+    block order.  Gather and both scatters against the oracle, both stack layouts."""
+    (H, W, C), bs, bst, bo, blocks = case
+    N = 2
+    rng = np.random.default_rng(len(blocks) + H)
+    x = rng.standard_normal((N, H, W, C)).astype(np.float32)
+    base = rng.standard_normal((N, H, W, C)).astype(np.float32)
+    idx = np.asarray(blocks, np.int16).reshape(-1, 3)
+    cnt = np.array([len(idx)], np.int32)
+    idx_d = dev(idx) if len(idx) else torch.zeros((1, 3), dtype=torch.int16, device=DEV)
+    idx_o = idx if len(idx) else np.zeros((1, 3), np.int16)
+    cnt_t = torch.from_numpy(cnt)
+    for transpose in (False, True):
+        g_o = orc.sparse_gather(x, cnt, idx_o, bs, bst, bo, transpose=transpose)
+        g = sbnet_amd.sparse_gather(dev(x), cnt_t, idx_d, bs, bst, bo, transpose=transpose)
+        assert tuple(g.shape) == g_o.shape
+        np.testing.assert_array_equal(host(g), g_o)
+        stack = rng.standard_normal(g_o.shape).astype(np.float32)
+        for add in (False, True):
+            y_o = orc.sparse_scatter(stack, cnt, idx_o, base, bs, bst, bo, add=add, transpose=transpose)
+            y = sbnet_amd.sparse_scatter(dev(stack), cnt_t, idx_d, dev(base), bs, bst, bo, add=add,
+                                         transpose=transpose)
+            np.testing.assert_array_equal(host(y), y_o)
+            bd = dev(base)
+            sbnet_amd.sparse_scatter_var(dev(stack), cnt_t, idx_d, bd, bs, bst, bo, add=add, transpose=transpose)
+            np.testing.assert_array_equal(host(bd), y_o)
+
+
 def test_reduce_mask_rows_past_count_untouched():
     mask = np.zeros((1, 8, 8, 1), np.float32)
     mask[0, 0, 0, 0] = 1.0
