@@ -1571,6 +1571,9 @@ static bool make_tile_args(const Geom& g, int numActive, int vec, TileArgs& a, i
     if (maxP < 1) return false;
     a.psplit = (RS + maxP - 1) / maxP;
     a.P = (RS + a.psplit - 1) / a.psplit;
+    // whole dwordx4 slots per planar run where the limits allow: only a plane's last split then ends in a
+    // partial slot
+    if (a.psplit > 1 && ((a.P + 3) & ~3) <= maxP) a.P = (a.P + 3) & ~3;
     a.psplit = (RS + a.P - 1) / a.P;
     a.Pp = (a.P + 31) / 32 * 32;
     a.vpr = (uint32_t)((a.P + 3) / 4);
