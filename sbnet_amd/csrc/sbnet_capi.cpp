@@ -50,7 +50,7 @@ HostSignal* host_signal()
     HostSignal& s = t_signal[dev];
     if (!s.host && !s.failed) {
         void* p = nullptr;
-        if (hipHostMalloc(&p, 64, hipHostMallocMapped) != hipSuccess || !p) {
+        if (hipHostMalloc(&p, 64, hipHostMallocMapped | hipHostMallocPortable) != hipSuccess || !p) {
             (void)hipGetLastError();
             s.failed = true;
         } else {
