@@ -4,6 +4,8 @@ device work (reduce_mask.cc:132-138; sparse_gather.cc:164-175, 307-327).  No ker
 import ctypes
 import os
 import re
+import shutil
+import subprocess
 
 import pytest
 
@@ -144,6 +146,22 @@ def test_scatter_rejects_aliasing_output():
     rc = lib.sbnet_sparse_scatter(FAKE, 1, FAKE, FAKE, dims, 4, ok, 2, ok, 2, ok, 2, 0, 0, 0,
                                   ctypes.c_void_p(0x1000 + 16), None, 0, None)
     assert rc == _lib.SBNET_EINVAL_ARG
+
+
+@pytest.mark.skipif(shutil.which("g++") is None, reason="needs a host C++ compiler")
+def test_reference_functor_header_compiles_links_and_reports_errors(tmp_path):
+    """include/sbnet_reference_functors.hpp gives the reference's functor templates (reduce_mask.h:23-44,
+    sparse_gather.h:23-76) their GPU specialisations on top of the C ABI.  tests/cxx/functor_shim_check.cpp uses it
+    as a build of the reference would and calls every functor with arguments the library rejects before any
+    device work."""
+    exe = str(tmp_path / "functor_shim_check")
+    libdir = os.path.dirname(_lib.LIB_PATH)
+    cmd = ["g++", "-std=c++14", "-Wall", "-Wextra", "-Werror", "-I", os.path.join(ROOT, "include"), "-o", exe,
+           os.path.join(ROOT, "tests", "cxx", "functor_shim_check.cpp"), "-L", libdir, "-lsbnet_amd",
+           "-Wl,-rpath," + libdir, "-Wl,-rpath,/opt/rocm/lib"]
+    subprocess.run(cmd, check=True, capture_output=True, text=True)
+    out = subprocess.run([exe], check=True, capture_output=True, text=True)
+    assert "functor shim ok" in out.stdout
 
 
 def test_python_mirror_fails_loudly_without_library(monkeypatch):
