@@ -479,7 +479,7 @@ int sbnet_timer_start(void* stream, int64_t* start_event)
     SBNET_HIP(hipEventCreate(&ev));
     hipError_t e = hipEventRecord(ev, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) {
-        hipEventDestroy(ev);
+        (void)hipEventDestroy(ev);
         return hip_fail(e);
     }
     *start_event = (int64_t)reinterpret_cast<intptr_t>(ev);
@@ -495,8 +495,8 @@ int sbnet_timer_end(int64_t start_event, void* stream, float* dt_ms)
     hipError_t e = hipEventRecord(end, static_cast<hipStream_t>(stream));
     if (e == hipSuccess) e = hipEventSynchronize(end);
     if (e == hipSuccess) e = hipEventElapsedTime(dt_ms, start, end);
-    hipEventDestroy(end);
-    hipEventDestroy(start);
+    (void)hipEventDestroy(end);
+    (void)hipEventDestroy(start);
     if (e != hipSuccess) return hip_fail(e);
     return SBNET_OK;
 }

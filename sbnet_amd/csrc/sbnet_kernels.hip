@@ -7,8 +7,9 @@
 //   * for the fused NHWC <-> [blocks, C, R, S] transpose, a tile of Ct channels x P block pixels
 //     staged through LDS so that both the NHWC side (runs of Ct floats per pixel) and the planar
 //     side (runs of P floats per channel) move in long contiguous pieces; the planar runs start
-//     at arbitrary 4-byte alignment (27x27 planes are 729 floats), so every run is split into a
-//     scalar head, an aligned dwordx4 body and a scalar tail;
+//     at arbitrary 4-byte alignment (27x27 planes are 729 floats): the scatter reads them as
+//     misaligned dwordx4 slots, the gather writes whole, aligned 128-byte lines;
+//   * raw buffer addressing with out-of-range offsets instead of branches around loads and stores;
 //   * several independent loads in flight per lane before the first use;
 //   * no integer division in inner loops (multiply-high reciprocals prepared on the host);
 //   * wave64 ballot / popcount for the ordered stream compaction of reduce_mask.
@@ -18,8 +19,6 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
-#include <stdlib.h>
-#include <string.h>
 
 #include "sbnet_launch.h"
 
@@ -1412,39 +1411,12 @@ static int ilog2_floor(uint32_t v)
     return l;
 }
 
-static uint32_t pow2_ceil(uint32_t v)
-{
-    uint32_t p = 1;
-    while (p < v) p <<= 1;
-    return p;
-}
-
 constexpr int GRID_Y_MAX = 65535;
 
 // One workgroup per tile, as (tiles per block, blocks) when the block count fits the y dimension of a launch.
 static dim3 tile_grid(int grid2d, uint32_t tpb, int numActive, uint32_t total)
 {
     return grid2d ? dim3(tpb, (unsigned)numActive) : dim3(total);
-}
-
-// Optional overrides for experiments: SBNET_TUNE="ct=32,lds=32768,wg=256,ps=3,lines=1".
-struct Tune {
-    int ct = 0, ldsBytes = 0, wg = 0, ps = 0, lines = -1, pad = 0;
-};
-
-static Tune read_tune()
-{
-    Tune t;
-    const char* s = getenv("SBNET_TUNE");
-    if (!s) return t;
-    const char* p;
-    if ((p = strstr(s, "ct="))) t.ct = atoi(p + 3);
-    if ((p = strstr(s, "lds="))) t.ldsBytes = atoi(p + 4);
-    if ((p = strstr(s, "wg="))) t.wg = atoi(p + 3);
-    if ((p = strstr(s, "ps="))) t.ps = atoi(p + 3);
-    if ((p = strstr(s, "lines="))) t.lines = atoi(p + 6);
-    if ((p = strstr(s, "pad="))) t.pad = atoi(p + 4);
-    return t;
 }
 
 static int pick_vec(const Geom& g, const void* a, const void* b)
@@ -1540,13 +1512,12 @@ static bool nhwc_fits_buffers(const Geom& g)
 static bool make_tile_args(const Geom& g, int numActive, int vec, TileArgs& a, int& threads, size_t& ldsBytes,
                            unsigned& grid, int defaultLdsBudget)
 {
-    static const Tune tune = read_tune();
     a.g = g;
     const int64_t RS64 = (int64_t)g.R * g.S;
     if (RS64 >= (1ll << 30)) return false;
     const int RS = (int)RS64;
     // channels per tile: 32 floats (one 128-byte line per pixel) unless C is smaller
-    const int ctWant = tune.ct > 0 ? tune.ct : 32;
+    const int ctWant = 32;
     int lpp = 1;
     while (lpp * 2 * vec <= ctWant && lpp * vec < g.C) lpp *= 2;
     a.Ct = lpp * vec;
@@ -1554,7 +1525,7 @@ static bool make_tile_args(const Geom& g, int numActive, int vec, TileArgs& a, i
     a.cchunks = (g.C + a.Ct - 1) / a.Ct;
     // Pixels per tile are bounded by the LDS budget and by the TILE_LD registers per thread that hold a
     // tile in flight on either side.  The smallest workgroup that takes a whole block plane wins.
-    const int budget = tune.ldsBytes > 0 ? tune.ldsBytes : defaultLdsBudget;
+    const int budget = defaultLdsBudget;
     int maxP = 0;
     threads = 0;
     for (int nthr = 64; nthr <= 512; nthr *= 2) {
@@ -1566,8 +1537,6 @@ static bool make_tile_args(const Geom& g, int numActive, int vec, TileArgs& a, i
         threads = nthr;
         if (maxP >= RS) break;
     }
-    if (tune.wg > 0 && tune.wg < threads) return false;  // experiments must pick a sufficient size
-    if (tune.wg > 0) threads = tune.wg;
     if (maxP < 1) return false;
     a.psplit = (RS + maxP - 1) / maxP;
     a.P = (RS + a.psplit - 1) / a.psplit;
@@ -1600,8 +1569,6 @@ static bool make_tile_args(const Geom& g, int numActive, int vec, TileArgs& a, i
 static bool make_line_args(const Geom& g, int numActive, const float* y, LineArgs& a, int& threads, int& ld,
                            size_t& ldsBytes, unsigned& grid)
 {
-    static const Tune tune = read_tune();
-    if (tune.lines == 0) return false;
     if (g.C % 4 != 0 || (reinterpret_cast<uintptr_t>(y) & 15) != 0) return false;
     a.g = g;
     const int64_t RS64 = (int64_t)g.R * g.S;
@@ -1629,8 +1596,6 @@ static bool make_line_args(const Geom& g, int numActive, const float* y, LineArg
         if (cap < 2 * LINE_FLOATS) return false;
         a.psplit = (RS + cap - 1) / cap;
     }
-    if (tune.ps > 0) a.psplit = tune.ps;
-    if (tune.wg > 0) threads = tune.wg;
     a.P = (RS + a.psplit - 1) / a.psplit;
     a.psplit = (RS + a.P - 1) / a.P;
     // A tile that takes whole planes writes one contiguous piece of y in k_gather_planar already.
@@ -1642,7 +1607,7 @@ static bool make_line_args(const Geom& g, int numActive, const float* y, LineArg
     if (ld < 4) ld = 4;
     if (ld > 8) return false;
     a.Pp = (win + 3 + 31) / 32 * 32;
-    ldsBytes = (size_t)a.Ct * a.Pp * sizeof(float) + (size_t)tune.pad;
+    ldsBytes = (size_t)a.Ct * a.Pp * sizeof(float);
     if (ldsBytes > 64 * 1024) return false;
     // slots per row: the written range of a row is at most P + LINE_EXT floats; when every chunk starts on a
     // line it is a whole number of lines
