@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the reduce_mask -> sparse_gather -> sparse_scatter path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--density 0.30] [--all-configs] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--density 0.30] [--all-configs] [--only C5] [--no-cpu]
 
 A step is one pass of the path over the LiDAR-BEV-shaped workload (x = [1,800,800,128] fp32,
 27x27 blocks, stride 25, offset -1, max pooling, tol 0.5, `--density` of the 1024 blocks active):
@@ -52,6 +52,9 @@ def parse():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--density", type=float, default=0.30)
     ap.add_argument("--all-configs", action="store_true")
+    ap.add_argument("--only", default=None, metavar="NAME",
+                    help="time one configuration only (C1, C2, C3@5%%, C3@15%%, C3@30%%, C4, C5) and print its row to "
+                         "stdout instead of the benchmark line: for profiling the other configurations' kernels")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline (profiling runs)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run the library's plain copy kernel on 256 MiB, 10 times: a kernel of known traffic "
@@ -338,6 +341,13 @@ def main():
         del src, dst
         torch.cuda.empty_cache()
 
+    if args.only:
+        if args.only not in CONFIGS:
+            print("bench.py: --only takes one of %s" % ", ".join(CONFIGS), file=sys.stderr)
+            sys.exit(2)
+        print(json.dumps(config_row(args.only, torch, lib, workloads)))
+        return
+
     wl = workloads.config3(args.density)
     path = Path(wl, torch, lib, nsets=3)
     nsets = len(path.sets)
@@ -444,29 +454,34 @@ def main():
     if args.all_configs:
         del path
         torch.cuda.empty_cache()
-        rows = []
-        gens = [("C1", workloads.config1, {}), ("C2", workloads.config2, {}),
-                ("C3@5%", workloads.config3, {"density": 0.05}), ("C3@15%", workloads.config3, {"density": 0.15}),
-                ("C3@30%", workloads.config3, {"density": 0.30}), ("C4", workloads.config4, {}),
-                ("C5", workloads.config5, {})]
-        for name, gen, kw in gens:
-            w = gen(**kw)
-            p = Path(w, torch, lib, nsets=2 if name == "C4" else 3)
-            n = len(p.sets)
-            for i in range(5):
-                p.step(i % n)
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            K = 50
-            for i in range(K):
-                p.step(i % n)
-            torch.cuda.synchronize()
-            e2e = (time.perf_counter() - t0) / K * 1e6
-            row = {"config": name, "M": p.M, "end_to_end_us": round(e2e, 1), "ops": p.op_table()}
-            rows.append(row)
-            print(json.dumps(row), file=sys.stderr)
-            del p
-            torch.cuda.empty_cache()
+        for name in CONFIGS:
+            print(json.dumps(config_row(name, torch, lib, workloads)), file=sys.stderr)
+
+
+CONFIGS = ["C1", "C2", "C3@5%", "C3@15%", "C3@30%", "C4", "C5"]
+
+
+def config_row(name, torch, lib, workloads):
+    """End-to-end time (host-visible count) and per-op device times of one configuration."""
+    gens = {"C1": (workloads.config1, {}), "C2": (workloads.config2, {}), "C3@5%": (workloads.config3, {"density": 0.05}),
+            "C3@15%": (workloads.config3, {"density": 0.15}), "C3@30%": (workloads.config3, {"density": 0.30}),
+            "C4": (workloads.config4, {}), "C5": (workloads.config5, {})}
+    gen, kw = gens[name]
+    p = Path(gen(**kw), torch, lib, nsets=2 if name == "C4" else 3)
+    n = len(p.sets)
+    for i in range(5):
+        p.step(i % n)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    K = 50
+    for i in range(K):
+        p.step(i % n)
+    torch.cuda.synchronize()
+    e2e = (time.perf_counter() - t0) / K * 1e6
+    row = {"config": name, "M": p.M, "end_to_end_us": round(e2e, 1), "ops": p.op_table()}
+    del p
+    torch.cuda.empty_cache()
+    return row
 
 
 if __name__ == "__main__":
