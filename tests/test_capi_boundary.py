@@ -149,17 +149,14 @@ def test_scatter_rejects_aliasing_output():
 
 
 @pytest.mark.skipif(shutil.which("g++") is None, reason="needs a host C++ compiler")
-def test_reference_functor_header_compiles_links_and_reports_errors(tmp_path):
+def test_reference_functor_header_compiles_links_and_reports_errors():
     """include/sbnet_reference_functors.hpp gives the reference's functor templates (reduce_mask.h:23-44,
     sparse_gather.h:23-76) their GPU specialisations on top of the C ABI.  tests/cxx/functor_shim_check.cpp uses it
     as a build of the reference would and calls every functor with arguments the library rejects before any
     device work."""
-    exe = str(tmp_path / "functor_shim_check")
-    libdir = os.path.dirname(_lib.LIB_PATH)
-    cmd = ["g++", "-std=c++14", "-Wall", "-Wextra", "-Werror", "-I", os.path.join(ROOT, "include"), "-o", exe,
-           os.path.join(ROOT, "tests", "cxx", "functor_shim_check.cpp"), "-L", libdir, "-lsbnet_amd",
-           "-Wl,-rpath," + libdir, "-Wl,-rpath,/opt/rocm/lib"]
-    subprocess.run(cmd, check=True, capture_output=True, text=True)
+    subprocess.run(["make", "-B", "-C", os.path.join(ROOT, "tests", "cxx"), "_build/functor_shim_check"], check=True,
+                   capture_output=True, text=True)
+    exe = os.path.join(ROOT, "tests", "cxx", "_build", "functor_shim_check")
     out = subprocess.run([exe], check=True, capture_output=True, text=True)
     assert "functor shim ok" in out.stdout
 

@@ -869,6 +869,18 @@ def test_random_geometries(seed):
 # functor-level entry points and the copy
 # ---------------------------------------------------------------------------------------------
 
+def test_reference_functors_in_cxx_against_the_oracle():
+    """tests/cxx/functor_shim_gpu.cpp drives reduce_mask -> sparse_gather -> copy + sparse_scatter through the
+    reference's functor templates, specialised by include/sbnet_reference_functors.hpp, and compares every result
+    with the CPU oracle bit for bit.  The program is built beforehand (make -C tests/cxx, part of build())."""
+    import subprocess
+    exe = os.path.join(HERE, "cxx", "_build", "functor_shim_gpu")
+    assert os.path.exists(exe), "tests/cxx/_build/functor_shim_gpu is missing: run make -C tests/cxx"
+    out = subprocess.run([exe], capture_output=True, text=True, timeout=100)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert "functor shim gpu ok" in out.stdout
+
+
 def test_functor_level_entry_points():
     import ctypes
     from sbnet_amd import _lib
