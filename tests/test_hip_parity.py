@@ -563,6 +563,34 @@ def test_edge_geometries(case):
             np.testing.assert_array_equal(host(bd), y_o)
 
 
+def test_reduce_mask_random_sweep():
+    """Seeded random reduce_mask problems: image and block sizes from 1 to ~90 / ~40, strides smaller and larger than
+    the blocks, offsets on either side of zero, block counts that under- and over-cover the image, binary, Gaussian
+    and wide-dynamic-range masks, both pooling modes, thresholds on either side of the data.  Count and ordered list
+    against the oracle."""
+    for seed in range(150):
+        rng = np.random.default_rng(10_000 + seed)
+        N, H, W = int(rng.integers(1, 5)), int(rng.integers(1, 90)), int(rng.integers(1, 90))
+        bs = (int(rng.integers(1, 40)), int(rng.integers(1, 40)))
+        bst = (int(rng.integers(1, 40)), int(rng.integers(1, 40)))
+        bo = (int(rng.integers(-20, 5)), int(rng.integers(-20, 5)))
+        bc = [int(rng.integers(1, 12)), int(rng.integers(1, 12))]
+        avg = bool(rng.integers(0, 2))
+        kind = int(rng.integers(0, 3))
+        if kind == 0:
+            mask = (rng.random((N, H, W, 1)) < rng.random() * 0.2).astype(np.float32)
+        elif kind == 1:
+            mask = rng.standard_normal((N, H, W, 1)).astype(np.float32)
+        else:
+            mask = (rng.standard_normal((N, H, W, 1)) * 10.0 ** rng.integers(-3, 4, (N, H, W, 1))).astype(np.float32)
+        tol = float(rng.choice([0.0, 0.05, 0.5, -0.1, float(np.percentile(mask, 90))]))
+        idx_o, cnt_o = orc.reduce_mask(mask, bc, bs, bst, bo, tol, avg)
+        r = sbnet_amd.reduce_mask(dev(mask), bc, bs, bst, bo, tol=tol, avgpool=avg)
+        M = int(cnt_o[0])
+        assert int(r.bin_counts[0]) == M, (seed, N, H, W, bs, bst, bo, bc, avg, kind, tol)
+        np.testing.assert_array_equal(host(r.active_block_indices)[:M], idx_o[:M], err_msg=str(seed))
+
+
 def test_reduce_mask_rows_past_count_untouched():
     mask = np.zeros((1, 8, 8, 1), np.float32)
     mask[0, 0, 0, 0] = 1.0
