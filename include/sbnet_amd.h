@@ -22,7 +22,9 @@
  *     reference's "should be one-dimensional with shape[0] == 2" check can be mirrored.
  *   - Every function returns an sbnet_status.  No function ever calls exit(); the reference
  *     prints and exits on a device error (op_utils.h:27-35), this library returns SBNET_EHIP.
- *   - Re-entrant: no global mutable state apart from a thread-local last-error slot.
+ *   - Re-entrant.  What the library keeps between calls: a thread-local last-error slot, one pinned
+ *     count word per thread and device (sbnet_reduce_mask with a host count), and the buffers of
+ *     sbnet_scratch_acquire for callers that use it; sbnet_shutdown frees the last two.
  */
 #ifndef SBNET_AMD_H
 #define SBNET_AMD_H
@@ -156,9 +158,9 @@ int sbnet_sparse_gather_functor(const float* x, int N, int H, int W, int C, floa
  * sparse_scatter / sparse_scatter_var
  * ---------------------------------------------------------------------------------------- */
 
-/* Bytes of scratch that let an overlapping atomic scatter-add run without atomics and that let sparse_scatter
-   build its output in one pass instead of copying ybase first (see workspace below); 0 when neither applies to
-   this geometry. */
+/* Bytes of scratch that let an overlapping atomic scatter-add run without atomics, that give overlapping plain
+   writes the CPU functor's order, and that let sparse_scatter build its output in one pass instead of copying
+   ybase first (see workspace below); 0 when none of these applies to this geometry. */
 size_t sbnet_sparse_scatter_workspace_bytes(int32_t num_active, const int64_t* ybase_dims, int ybase_rank,
                                             const int32_t* bsize, int bsize_len,
                                             const int32_t* bstride, int bstride_len,
@@ -176,10 +178,16 @@ size_t sbnet_sparse_scatter_workspace_bytes(int32_t num_active, const int64_t* y
  *   y           device fp32, same shape, must not overlap ybase
  *   Pixels of a block that fall outside the image are dropped (sparse_gather.cc:121).
  *   add=1, atomic=0 requires bstride >= bsize on both axes (sparse_gather.cc:322-326).
- *   add=0 with overlapping blocks: as in the reference's GPU path, which block wins on an
- *   overlapped pixel is unspecified unless the overlapping values are equal.
+ *   add=0 with overlapping blocks (bstride < bsize): the reference's CPU functor walks the list front to
+ *   back, so the block listed last wins on a pixel that several blocks cover (sparse_gather.cc:105-129).
+ *   Given scratch (below) this library writes exactly that, for both stack layouts and for lists that name
+ *   a block twice.  Without scratch, as in the reference's GPU path, which block wins is unspecified unless
+ *   the overlapping values are equal.
  *   workspace   optional device scratch (4-byte aligned) of sbnet_sparse_scatter_workspace_bytes() bytes,
- *               or NULL.  Two uses.
+ *               or NULL.  Three uses.
+ *               (0) add=0 and bstride < bsize: an owner map (one int32 per pixel: the last listed block that
+ *               covers it) is built first and every block writes only the pixels it owns: the CPU functor's
+ *               result, no pixel written twice.
  *               (1) sbnet_sparse_scatter with atomic=0: when the blocks cover 16 MB or more, y is built from
  *               two disjoint parts instead of "copy ybase, scatter on top": pixels that no active block covers
  *               are copied from ybase, covered ones are written by the scatter, which reads ybase where it
@@ -221,6 +229,28 @@ int sbnet_sparse_scatter_functor(const float* x, int N, int H, int W, int C, flo
                                  int bOffsH0, int bOffsW0, int bSzH, int bSzW, int bStrH,
                                  int bStrW, int numActive, const int16_t* activeBlockIndices,
                                  int add, int transpose, int atomic, void* stream);
+
+/* The same with scratch (sbnet_sparse_scatter_workspace_bytes(), as for the op level): overlapping atomic adds run
+   without atomics and overlapping plain writes follow the CPU functor's order.  No counterpart in the reference,
+   whose functor has no scratch argument; include/sbnet_reference_functors.hpp calls this one with scratch from
+   its scratch provider. */
+int sbnet_sparse_scatter_functor_ws(const float* x, int N, int H, int W, int C, float* y,
+                                    int bOffsH0, int bOffsW0, int bSzH, int bSzW, int bStrH,
+                                    int bStrW, int numActive, const int16_t* activeBlockIndices,
+                                    int add, int transpose, int atomic,
+                                    void* workspace, size_t workspace_bytes, void* stream);
+
+/* Library-managed device scratch for callers that have no allocator at hand (the functor level of the reference
+   passes none down, sparse_gather.h:45-66): returns a buffer of at least `bytes` bytes on the current device that
+   stays valid until the next sbnet_scratch_acquire on the same stream or sbnet_shutdown.  One grow-only buffer is
+   kept per (device, stream); calls on one stream run in order, so they may share it.  Growing allocates (and
+   waits for the stream); a request that would have to grow while `stream` is being captured returns NULL, as does
+   a failed allocation.  Thread-safe. */
+void* sbnet_scratch_acquire(size_t bytes, void* stream);
+
+/* Frees what the library keeps between calls: the buffers of sbnet_scratch_acquire and the pinned count words of
+   threads that have ended.  Optional; waits for the device.  The library can be used again afterwards. */
+int sbnet_shutdown(void);
 
 /* Replaces CopyTensorFunctor<GPUDevice,float>::operator() (sparse_gather.h:69-76,
    sparse_gather.cu:268-276) without its stream synchronisation.  count is in floats. */

@@ -17,7 +17,7 @@
  *     SBNET_AMD_GPU_FUNCTORS(GPUDevice)
  *
  * replaces both .cu files and the OpKernels compile unchanged.  `Device` only has to offer stream(), returning
- * the HIP stream the op must run on (Eigen::GpuDevice does).  The primary templates must be declared before
+ * a reference to the HIP stream the op must run on (Eigen::GpuDevice does; getStream hands out its address).  The primary templates must be declared before
  * the macro is used; this header does not declare them.
  *
  * Differences from the .cu files it replaces, all inherited from the library: block indices come out in
@@ -28,6 +28,8 @@
 #ifndef SBNET_REFERENCE_FUNCTORS_HPP
 #define SBNET_REFERENCE_FUNCTORS_HPP
 
+#include <cstddef>
+#include <cstdint>
 #include <cstdio>
 #include <cstdlib>
 
@@ -57,6 +59,24 @@ inline void check(int status, const char* what)
 
 template <typename Device> inline void* stream_of(const Device& d) { return (void*)d.stream(); }
 
+// Device scratch for the functors.  The reference's functor signatures carry no scratch, but the fast paths of
+// the library need some (reduce_mask's flags; the atomic-free overlapping scatter-add; ordered overlapping
+// writes).  A provider returns at least `bytes` bytes valid until its next call on the same stream, or NULL
+// (the functors then take the paths that need none).  The default is the library's own per-stream buffer; a
+// framework with a stream-ordered allocator can install its own.
+typedef void* (*ScratchProvider)(size_t bytes, void* stream);
+
+inline ScratchProvider& scratch_provider()
+{
+    static ScratchProvider p = sbnet_scratch_acquire;
+    return p;
+}
+
+inline void* scratch(size_t bytes, void* stream)
+{
+    return (bytes && scratch_provider()) ? scratch_provider()(bytes, stream) : NULL;
+}
+
 }  // namespace sbnet_amd
 
 #define SBNET_AMD_GPU_FUNCTORS(DEVICE)                                                                              \
@@ -66,11 +86,14 @@ template <typename Device> inline void* stream_of(const Device& d) { return (voi
                         unsigned int numBins, unsigned int binSize, short* activeBlockIndices, int* binCounts,      \
                         bool avgPool)                                                                               \
         {                                                                                                           \
-            /* no workspace: the library allocates and frees one per call; bind the op level for speed */          \
+            const int32_t bcount_[2] = {bCntH, bCntW};                                                              \
+            const size_t need_ = sbnet_reduce_mask_workspace_bytes(N, bcount_, 2);                                  \
+            void* ws_ = sbnet_amd::scratch(need_, sbnet_amd::stream_of(d));                                         \
+            /* without scratch the library allocates and frees its own for the call */                              \
             sbnet_amd::check(sbnet_reduce_mask_functor(mask, N, H, W, threshold, bOffsH0, bOffsW0, bSzH, bSzW,      \
                                                        bStrH, bStrW, bCntH, bCntW, numBins, binSize,                \
-                                                       activeBlockIndices, binCounts, avgPool ? 1 : 0, NULL, 0,     \
-                                                       sbnet_amd::stream_of(d)),                                    \
+                                                       activeBlockIndices, binCounts, avgPool ? 1 : 0, ws_,         \
+                                                       ws_ ? need_ : 0, sbnet_amd::stream_of(d)),                   \
                              "ReduceMaskFunctor");                                                                  \
         }                                                                                                           \
     };                                                                                                              \
@@ -90,10 +113,19 @@ template <typename Device> inline void* stream_of(const Device& d) { return (voi
                         int bSzH, int bSzW, int bStrH, int bStrW, int numActive, const short* activeBlockIndices,   \
                         bool add, bool transpose, bool atomic)                                                      \
         {                                                                                                           \
-            sbnet_amd::check(sbnet_sparse_scatter_functor(x, N, H, W, C, y, bOffsH0, bOffsW0, bSzH, bSzW, bStrH,    \
-                                                          bStrW, numActive, activeBlockIndices, add ? 1 : 0,        \
-                                                          transpose ? 1 : 0, atomic ? 1 : 0,                        \
-                                                          sbnet_amd::stream_of(d)),                                 \
+            size_t need_ = 0;                                                                                       \
+            if ((add && atomic) || (!add && (bStrH < bSzH || bStrW < bSzW))) {                                      \
+                const int64_t dims_[4] = {N, H, W, C};                                                              \
+                const int32_t bsize_[2] = {bSzH, bSzW}, bstride_[2] = {bStrH, bStrW},                               \
+                              boffset_[2] = {bOffsH0, bOffsW0};                                                     \
+                need_ = sbnet_sparse_scatter_workspace_bytes(numActive, dims_, 4, bsize_, 2, bstride_, 2,           \
+                                                             boffset_, 2);                                          \
+            }                                                                                                       \
+            void* ws_ = sbnet_amd::scratch(need_, sbnet_amd::stream_of(d));                                         \
+            sbnet_amd::check(sbnet_sparse_scatter_functor_ws(x, N, H, W, C, y, bOffsH0, bOffsW0, bSzH, bSzW,        \
+                                                             bStrH, bStrW, numActive, activeBlockIndices,           \
+                                                             add ? 1 : 0, transpose ? 1 : 0, atomic ? 1 : 0, ws_,   \
+                                                             ws_ ? need_ : 0, sbnet_amd::stream_of(d)),             \
                              "SparseScatterFunctor");                                                               \
         }                                                                                                           \
     };                                                                                                              \
@@ -103,6 +135,8 @@ template <typename Device> inline void* stream_of(const Device& d) { return (voi
             sbnet_amd::check(sbnet_copy_tensor(dst, src, (size_t)count, sbnet_amd::stream_of(d)),                   \
                              "CopyTensorFunctor");                                                                  \
         }                                                                                                           \
+        /* sparse_gather.h:75, sparse_gather.cu:275: the address of the device's stream handle */                   \
+        auto getStream(const DEVICE& d) -> decltype(&d.stream()) { return &d.stream(); }                            \
     };                                                                                                              \
     template struct ReduceMaskFunctor<DEVICE, float>;                                                               \
     template struct SparseGatherFunctor<DEVICE, float>;                                                             \

@@ -53,6 +53,10 @@ SIGNATURES = {
                                                  _i32p, _int, _int, _int, _int, _vp, _vp, _sz, _vp]),
     "sbnet_sparse_scatter_var_device_count": (_int, [_vp, _vp, _i32, _vp, _vp, _i64p, _int, _i32p, _int, _i32p, _int,
                                                      _i32p, _int, _int, _int, _int, _vp, _sz, _vp]),
+    "sbnet_sparse_scatter_functor_ws": (_int, [_vp, _int, _int, _int, _int, _vp] + [_int] * 7 + [_vp, _int, _int,
+                                                                                                 _int, _vp, _sz, _vp]),
+    "sbnet_scratch_acquire": (_vp, [_sz, _vp]),
+    "sbnet_shutdown": (_int, []),
     "sbnet_copy_tensor": (_int, [_vp, _vp, _sz, _vp]),
     "sbnet_timer_start": (_int, [_vp, ctypes.POINTER(ctypes.c_int64)]),
     "sbnet_timer_end": (_int, [ctypes.c_int64, _vp, ctypes.POINTER(ctypes.c_float)]),

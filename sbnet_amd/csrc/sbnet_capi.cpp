@@ -9,6 +9,10 @@
 #include "../../include/sbnet_amd.h"
 
 #include <hip/hip_runtime_api.h>
+#include <sched.h>
+
+#include <mutex>
+#include <vector>
 
 #include "sbnet_launch.h"
 
@@ -41,24 +45,57 @@ struct HostSignal {
     uint32_t seq = 0;
     bool failed = false;                 // allocation refused once: do not try again
 };
-thread_local HostSignal t_signal[MAX_SIGNAL_DEVICES];
+
+// Words are handed out per thread and device; a thread that ends returns its words to a free list, so the
+// number of words is bounded by the largest number of threads alive at once, and sbnet_shutdown() frees
+// them.  Nothing is freed from a static destructor: the HIP runtime may already be gone by then.
+std::mutex g_signalMutex;
+std::vector<unsigned long long*> g_signalFree[MAX_SIGNAL_DEVICES];
+std::vector<unsigned long long*> g_signalAll;
+
+struct ThreadSignals {
+    HostSignal dev[MAX_SIGNAL_DEVICES];
+    ~ThreadSignals()
+    {
+        std::lock_guard<std::mutex> lock(g_signalMutex);
+        for (int d = 0; d < MAX_SIGNAL_DEVICES; ++d)
+            if (dev[d].host) g_signalFree[d].push_back(dev[d].host);
+    }
+};
+thread_local ThreadSignals t_signal;
 
 HostSignal* host_signal()
 {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_SIGNAL_DEVICES) return nullptr;
-    HostSignal& s = t_signal[dev];
+    HostSignal& s = t_signal.dev[dev];
     if (!s.host && !s.failed) {
-        void* p = nullptr;
-        if (hipHostMalloc(&p, 64, hipHostMallocMapped | hipHostMallocPortable) != hipSuccess || !p) {
-            (void)hipGetLastError();
-            s.failed = true;
+        std::lock_guard<std::mutex> lock(g_signalMutex);
+        if (!g_signalFree[dev].empty()) {
+            s.host = g_signalFree[dev].back();
+            g_signalFree[dev].pop_back();
+            // the word keeps the last tag its previous owner saw: continue from there, never reuse a tag
+            s.seq = (uint32_t)(__atomic_load_n(s.host, __ATOMIC_ACQUIRE) >> 32);
         } else {
-            s.host = static_cast<unsigned long long*>(p);
-            *s.host = 0;
+            void* p = nullptr;
+            if (hipHostMalloc(&p, 64, hipHostMallocMapped | hipHostMallocPortable) != hipSuccess || !p) {
+                (void)hipGetLastError();
+                s.failed = true;
+            } else {
+                s.host = static_cast<unsigned long long*>(p);
+                *s.host = 0;
+                g_signalAll.push_back(s.host);
+            }
         }
     }
     return s.host ? &s : nullptr;
+}
+
+inline void cpu_relax()
+{
+#if defined(__x86_64__) || defined(__i386__)
+    __builtin_ia32_pause();
+#endif
 }
 
 // Waits until the word carries `seq` and returns the count; gives up (false) as soon as the stream has
@@ -66,12 +103,16 @@ HostSignal* host_signal()
 bool poll_host_signal(const HostSignal& s, uint32_t seq, hipStream_t stream, int32_t* count, hipError_t* err)
 {
     *err = hipSuccess;
+    // Back-off: the count normally arrives within a few microseconds, so the first reads only pause the core;
+    // behind a long queue the thread yields between reads instead of burning its core.
     for (uint32_t spins = 1;; ++spins) {
         const unsigned long long v = __atomic_load_n(s.host, __ATOMIC_ACQUIRE);
         if ((uint32_t)(v >> 32) == seq) {
             *count = (int32_t)(uint32_t)v;
             return true;
         }
+        if (spins < 4096u) cpu_relax();
+        else sched_yield();
         if ((spins & 255u) == 0) {
             const hipError_t q = hipStreamQuery(stream);
             if (q == hipErrorNotReady) {
@@ -228,9 +269,27 @@ int scatter_impl(const float* x, int32_t numActive, const int32_t* countDev, con
                                                 stream, done));
         if (done) return SBNET_OK;
     }
+    if (mode == sbnet::SCATTER_ASSIGN && workspace) {
+        // with scratch, overlapping plain writes land in the CPU functor's order (the block listed last wins)
+        bool done = false;
+        SBNET_HIP(sbnet::launch_scatter_owned(x, out, idx, numActive, g, transpose != 0, workspace, workspaceBytes,
+                                              stream, done));
+        if (done) return SBNET_OK;
+    }
     SBNET_HIP(sbnet::launch_scatter(x, out, idx, numActive, g, transpose != 0, mode, stream));
     return SBNET_OK;
 }
+
+// Library-managed scratch for callers without an allocator at hand (sbnet_scratch_acquire): one grow-only buffer
+// per (device, stream).  Work on one stream runs in order, so consecutive calls on that stream may share it.
+struct ScratchSlot {
+    int dev;
+    hipStream_t stream;
+    void* ptr;
+    size_t bytes;
+};
+std::mutex g_scratchMutex;
+std::vector<ScratchSlot> g_scratch;
 
 }  // namespace
 
@@ -348,8 +407,10 @@ size_t sbnet_sparse_scatter_workspace_bytes(int32_t num_active, const int64_t* y
     const size_t pull = sbnet::scatter_pull_workspace_bytes(g, num_active);
     const size_t color = sbnet::scatter_color_workspace_bytes(g, num_active);
     const size_t cover = sbnet::scatter_cover_workspace_bytes(g, num_active);
-    const size_t m = pull > color ? pull : color;
-    return m > cover ? m : cover;
+    const size_t owner = sbnet::scatter_owner_workspace_bytes(g, num_active);
+    size_t m = pull > color ? pull : color;
+    if (cover > m) m = cover;
+    return owner > m ? owner : m;
 }
 
 static int scatter_op(const float* x, int32_t num_active, const int32_t* bin_counts_device,
@@ -459,10 +520,95 @@ int sbnet_sparse_scatter_functor(const float* x, int N, int H, int W, int C, flo
                                  const int16_t* activeBlockIndices, int add, int transpose, int atomic,
                                  void* stream)
 {
+    return sbnet_sparse_scatter_functor_ws(x, N, H, W, C, y, bOffsH0, bOffsW0, bSzH, bSzW, bStrH, bStrW, numActive,
+                                           activeBlockIndices, add, transpose, atomic, nullptr, 0, stream);
+}
+
+int sbnet_sparse_scatter_functor_ws(const float* x, int N, int H, int W, int C, float* y, int bOffsH0,
+                                    int bOffsW0, int bSzH, int bSzW, int bStrH, int bStrW, int numActive,
+                                    const int16_t* activeBlockIndices, int add, int transpose, int atomic,
+                                    void* workspace, size_t workspace_bytes, void* stream)
+{
     const int32_t bsize[2] = {bSzH, bSzW}, bstride[2] = {bStrH, bStrW}, boffset[2] = {bOffsH0, bOffsW0};
     const int64_t dims[4] = {N, H, W, C};
     return scatter_impl(x, numActive, nullptr, activeBlockIndices, y, dims, bsize, bstride, boffset, add, atomic,
-                        transpose, nullptr, 0, static_cast<hipStream_t>(stream));
+                        transpose, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+void* sbnet_scratch_acquire(size_t bytes, void* stream)
+{
+    if (bytes == 0) return nullptr;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    std::lock_guard<std::mutex> lock(g_scratchMutex);
+    ScratchSlot* slot = nullptr;
+    for (ScratchSlot& c : g_scratch)
+        if (c.dev == dev && c.stream == s) slot = &c;
+    if (slot && slot->bytes >= bytes) return slot->ptr;
+    // growing allocates, which a stream under capture must not do
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &cap) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    if (cap != hipStreamCaptureStatusNone) return nullptr;
+    size_t want = (size_t)1 << 20;
+    while (want < bytes) want <<= 1;
+    void* p = nullptr;
+    if (hipMalloc(&p, want) != hipSuccess || !p) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    if (slot) {
+        // the old buffer may still be in use by work queued on the stream
+        (void)hipStreamSynchronize(s);
+        (void)hipFree(slot->ptr);
+        slot->ptr = p;
+        slot->bytes = want;
+    } else {
+        g_scratch.push_back(ScratchSlot{dev, s, p, want});
+    }
+    return p;
+}
+
+int sbnet_shutdown(void)
+{
+    hipError_t first = hipSuccess;
+    {
+        std::lock_guard<std::mutex> lock(g_scratchMutex);
+        for (ScratchSlot& c : g_scratch) {
+            int cur = 0;
+            (void)hipGetDevice(&cur);
+            (void)hipSetDevice(c.dev);
+            hipError_t e = hipFree(c.ptr);  // waits for the device
+            (void)hipSetDevice(cur);
+            if (e != hipSuccess && first == hipSuccess) first = e;
+        }
+        g_scratch.clear();
+    }
+    {
+        // only the words no thread holds; a live thread keeps its own until it ends
+        std::lock_guard<std::mutex> lock(g_signalMutex);
+        for (int d = 0; d < MAX_SIGNAL_DEVICES; ++d) {
+            for (unsigned long long* w : g_signalFree[d]) {
+                hipError_t e = hipHostFree(w);
+                if (e != hipSuccess && first == hipSuccess) first = e;
+                for (size_t i = 0; i < g_signalAll.size(); ++i)
+                    if (g_signalAll[i] == w) {
+                        g_signalAll[i] = g_signalAll.back();
+                        g_signalAll.pop_back();
+                        break;
+                    }
+            }
+            g_signalFree[d].clear();
+        }
+    }
+    if (first != hipSuccess) return hip_fail(first);
+    return SBNET_OK;
 }
 
 int sbnet_copy_tensor(float* dst, const float* src, size_t count, void* stream)

@@ -176,9 +176,17 @@ __device__ __forceinline__ bool beyond_count(const Geom& g, uint32_t ib)
 // detects that (`dup`), and then pass 0 handles every block with atomics and the other passes do nothing.
 constexpr int SCATTER_COLOR = 3;  // kernel-side mode; callers ask for SCATTER_ATOMIC
 
+// Plain writes ("=") of overlapping blocks in the sequential CPU functor's order: that functor visits the
+// list front to back (sparse_gather.cc:105), so on a pixel that several blocks cover the one listed last
+// wins.  A per-pixel owner map (the highest list position that covers the pixel, built by k_owner_fill and
+// k_owner_mark before the launch) lets every block write only the pixels it owns: no pixel is written twice,
+// and a block listed twice is handled like any other overlap.
+constexpr int SCATTER_OWNED = 4;  // kernel-side mode; callers ask for SCATTER_ASSIGN and give scratch
+
 struct ColorArgs {
     int kh, kw, pass;
     const int32_t* dup;
+    const int32_t* owner;  // SCATTER_OWNED: [N, H, W] list positions, -1 where no block covers the pixel
 };
 
 // True when this launch has nothing to do for the block; `atomics` tells how to add otherwise.
@@ -210,7 +218,7 @@ struct NhwcArgs {
     uint32_t blockV;  // vectors per block, R*rowV
     uint32_t cpb;     // chunks per block
     uint32_t units;   // numActive * cpb
-    FastDiv dCpb, dRow;
+    FastDiv dCpb, dRow, dCV;  // dCV: by the vectors per pixel, C/VEC
 };
 
 // sparse_gather.cc:67-88 with transpose == false.
@@ -295,7 +303,11 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc_wide(const float* __restri
             const int hh = o.h0 + (int)r;
             if ((unsigned)hh < (unsigned)a.g.H && j >= lo && j < hi) {
                 dst[u] = (((int64_t)o.n * a.g.H + hh) * a.g.W + o.w0) * CV + j;
-                v[u] = ld_stream(xb + e);
+                if (MODE == SCATTER_OWNED &&
+                    col.owner[((int64_t)o.n * a.g.H + hh) * a.g.W + o.w0 + (int)fdiv((uint32_t)j, a.dCV)] != (int32_t)ib)
+                    dst[u] = -1;
+                else
+                    v[u] = ld_stream(xb + e);
             }
         }
     }
@@ -307,7 +319,7 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc_wide(const float* __restri
 #pragma unroll
         for (int u = 0; u < NHWC_UNR; ++u)
             if (dst[u] >= 0) st_stream(yv + dst[u], vadd(cur[u], v[u]));
-    } else if (MODE == SCATTER_ASSIGN) {
+    } else if (MODE == SCATTER_ASSIGN || MODE == SCATTER_OWNED) {
 #pragma unroll
         for (int u = 0; u < NHWC_UNR; ++u)
             if (dst[u] >= 0) commit<VEC, SCATTER_ASSIGN>(yv + dst[u], v[u]);
@@ -526,6 +538,9 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
     const uint32_t e0 = chunk * NHWC_CHUNK + lane;
     vec v[NHWC_UNR];
     uint32_t dst[NHWC_UNR];
+    int32_t own[NHWC_UNR];
+    const rsrc_t wr = make_rsrc(MODE == SCATTER_OWNED ? col.owner + (int64_t)o.n * a.g.H * a.g.W : nullptr,
+                                MODE == SCATTER_OWNED ? (uint32_t)(a.g.H * a.g.W) * 4u : 0u);
 #pragma unroll
     for (int u = 0; u < NHWC_UNR; ++u) {
         const uint32_t e = e0 + u * 64;
@@ -536,8 +551,16 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
         dst[u] = ok ? (((uint32_t)hh * (uint32_t)a.g.W + (uint32_t)o.w0) * (uint32_t)CV + (uint32_t)j) * (uint32_t)(VEC * 4)
                     : BUF_OOB;
         v[u] = buf_load<VEC>(xr, ok ? e * (uint32_t)(VEC * 4) : BUF_OOB);  // off-image parts are not read
+        if (MODE == SCATTER_OWNED) {
+            const uint32_t pix = (uint32_t)hh * (uint32_t)a.g.W + (uint32_t)o.w0 + fdiv((uint32_t)j, a.dCV);
+            own[u] = __builtin_bit_cast(int32_t, buf_load<1>(wr, ok ? pix * 4u : BUF_OOB));
+        }
     }
-    if (MODE == SCATTER_ASSIGN) {
+    if (MODE == SCATTER_OWNED) {
+        // (an out-of-range owner read returns 0, which may equal ib: dst is BUF_OOB there already)
+#pragma unroll
+        for (int u = 0; u < NHWC_UNR; ++u) buf_store<BUF_NT>(yr, own[u] == (int32_t)ib ? dst[u] : BUF_OOB, v[u]);
+    } else if (MODE == SCATTER_ASSIGN) {
 #pragma unroll
         for (int u = 0; u < NHWC_UNR; ++u) buf_store<BUF_NT>(yr, dst[u], v[u]);
     } else if (MODE == SCATTER_ADD || (MODE == SCATTER_COLOR && !atomics)) {
@@ -560,7 +583,8 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
 
 // NHWC side of a tile: thread tid owns channel vector cl = tid & (lpp-1) of pixels pl0 + u*step,
 // u = 0 .. TILE_LD-1, pl0 = tid >> lppLog, step = nthr >> lppLog.  Walks those pixels keeping (r, s) by
-// increments and hands each one's byte offset inside the image (or BUF_OOB) to `f(u, pl, off)`.
+// increments and hands each one's byte offset inside the image (or BUF_OOB) and its pixel number h*W + w (only
+// meaningful with an in-range offset) to `f(u, pl, off, pix)`.
 template <int VEC, typename F>
 __device__ __forceinline__ void nhwc_walk(const TileArgs& a, const TileId& t, const BlockOrigin& o, uint32_t tid,
                                           uint32_t nthr, F f)
@@ -578,7 +602,7 @@ __device__ __forceinline__ void nhwc_walk(const TileArgs& a, const TileId& t, co
         const int hh = o.h0 + (int)r, ww = o.w0 + (int)s;
         const bool ok = cok && pl < (uint32_t)t.Pn && (unsigned)hh < (unsigned)a.g.H && (unsigned)ww < (unsigned)a.g.W;
         const uint32_t off = (((uint32_t)hh * (uint32_t)a.g.W + (uint32_t)ww) * (uint32_t)a.g.C + (uint32_t)c) * 4u;
-        f(u, pl, ok ? off : BUF_OOB);
+        f(u, pl, ok ? off : BUF_OOB, (uint32_t)hh * (uint32_t)a.g.W + (uint32_t)ww);
         pl += step;
         r += stepR;
         s += stepS;
@@ -608,7 +632,7 @@ __global__ __launch_bounds__(512) void k_gather_planar(const float* __restrict__
 
     vec v[TILE_LD];
     uint32_t pls[TILE_LD];
-    nhwc_walk<VEC>(a, t, o, tid, nthr, [&](int u, uint32_t pl, uint32_t off) {
+    nhwc_walk<VEC>(a, t, o, tid, nthr, [&](int u, uint32_t pl, uint32_t off, uint32_t) {
         v[u] = buf_load<VEC>(xr, off);
         pls[u] = pl;
     });
@@ -893,30 +917,39 @@ __global__ __launch_bounds__(512) void k_scatter_planar(const float* __restrict_
     const rsrc_t xr = make_rsrc(x + ((int64_t)t.ib * a.g.C + t.c0) * RS + t.p0,
                                 ((uint32_t)(t.ctEff - 1) * RS + (uint32_t)t.Pn) * 4u);
     const uint32_t slots = (uint32_t)t.ctEff * a.vpr;
-    f4 val[TILE_LD];
+    if (t.Pn >= 4) {
+        f4 val[TILE_LD];
 #pragma unroll
-    for (int u = 0; u < TILE_LD; ++u) {
-        const uint32_t i = u * nthr + tid;
-        const uint32_t c = fdiv(i, a.dVpr);
-        const int e0 = min(4 * (int)(i - c * a.vpr), t.Pn - 4);
-        val[u] = buf_load<4>(xr, (i < slots && e0 >= 0) ? (c * RS + (uint32_t)e0) * 4u : BUF_OOB);
-    }
-#pragma unroll
-    for (int u = 0; u < TILE_LD; ++u) {
-        const uint32_t i = u * nthr + tid;
-        if (i < slots) {
+        for (int u = 0; u < TILE_LD; ++u) {
+            const uint32_t i = u * nthr + tid;
             const uint32_t c = fdiv(i, a.dVpr);
-            const int e0 = 4 * (int)(i - c * a.vpr);
-            float* __restrict__ row = lds + c * a.Pp;
-            if (e0 + 4 <= t.Pn) {
-                *reinterpret_cast<f4*>(row + ((uint32_t)e0 ^ lds_swz(c))) = val[u];
-            } else if (e0 < t.Pn) {  // partial last slot: holds floats [Pn-4, Pn) of the run
-                const uint32_t t0 = (uint32_t)(t.Pn - 4);
-                row[(t0 + 0) ^ lds_swz(c)] = val[u].x;
-                row[(t0 + 1) ^ lds_swz(c)] = val[u].y;
-                row[(t0 + 2) ^ lds_swz(c)] = val[u].z;
-                row[(t0 + 3) ^ lds_swz(c)] = val[u].w;
+            const int e0 = min(4 * (int)(i - c * a.vpr), t.Pn - 4);
+            val[u] = buf_load<4>(xr, i < slots ? (c * RS + (uint32_t)e0) * 4u : BUF_OOB);
+        }
+#pragma unroll
+        for (int u = 0; u < TILE_LD; ++u) {
+            const uint32_t i = u * nthr + tid;
+            if (i < slots) {
+                const uint32_t c = fdiv(i, a.dVpr);
+                const int e0 = 4 * (int)(i - c * a.vpr);
+                float* __restrict__ row = lds + c * a.Pp;
+                if (e0 + 4 <= t.Pn) {
+                    *reinterpret_cast<f4*>(row + ((uint32_t)e0 ^ lds_swz(c))) = val[u];
+                } else if (e0 < t.Pn) {  // partial last slot: holds floats [Pn-4, Pn) of the run
+                    const uint32_t t0 = (uint32_t)(t.Pn - 4);
+                    row[(t0 + 0) ^ lds_swz(c)] = val[u].x;
+                    row[(t0 + 1) ^ lds_swz(c)] = val[u].y;
+                    row[(t0 + 2) ^ lds_swz(c)] = val[u].z;
+                    row[(t0 + 3) ^ lds_swz(c)] = val[u].w;
+                }
             }
+        }
+    } else {
+        // A plane's last split can hold fewer pixels than one slot (the split width is rounded up to whole slots,
+        // and 1-3 pixels may remain): one thread per row moves them float by float.
+        if (tid < (uint32_t)t.ctEff) {
+            for (int k = 0; k < t.Pn; ++k)
+                lds[tid * a.Pp + ((uint32_t)k ^ lds_swz(tid))] = buf_load<1>(xr, (tid * RS + (uint32_t)k) * 4u);
         }
     }
     lds_barrier();
@@ -930,8 +963,12 @@ __global__ __launch_bounds__(512) void k_scatter_planar(const float* __restrict_
     const uint32_t c0l = (tid & ((1u << a.lppLog) - 1u)) * VEC;
     vec w[TILE_LD];
     uint32_t offs[TILE_LD];
-    nhwc_walk<VEC>(a, t, o, tid, nthr, [&](int u, uint32_t pl, uint32_t off) {
+    int32_t own[TILE_LD];
+    const rsrc_t wr = make_rsrc(MODE == SCATTER_OWNED ? col.owner + (int64_t)o.n * a.g.H * a.g.W : nullptr,
+                                MODE == SCATTER_OWNED ? (uint32_t)(a.g.H * a.g.W) * 4u : 0u);
+    nhwc_walk<VEC>(a, t, o, tid, nthr, [&](int u, uint32_t pl, uint32_t off, uint32_t pix) {
         offs[u] = off;
+        if (MODE == SCATTER_OWNED) own[u] = __builtin_bit_cast(int32_t, buf_load<1>(wr, off != BUF_OOB ? pix * 4u : BUF_OOB));
         w[u] = vzero<VEC>();
         if (off != BUF_OOB) {
 #pragma unroll
@@ -941,7 +978,10 @@ __global__ __launch_bounds__(512) void k_scatter_planar(const float* __restrict_
             }
         }
     });
-    if (MODE == SCATTER_ASSIGN) {
+    if (MODE == SCATTER_OWNED) {
+#pragma unroll
+        for (int u = 0; u < TILE_LD; ++u) buf_store<BUF_NT>(yr, own[u] == (int32_t)t.ib ? offs[u] : BUF_OOB, w[u]);
+    } else if (MODE == SCATTER_ASSIGN) {
 #pragma unroll
         for (int u = 0; u < TILE_LD; ++u) buf_store<BUF_NT>(yr, offs[u], w[u]);
     } else if (MODE == SCATTER_ADD || (MODE == SCATTER_COLOR && !atomics)) {
@@ -967,7 +1007,8 @@ __global__ __launch_bounds__(512) void k_scatter_planar(const float* __restrict_
 // threads, so the NHWC side stays coalesced.
 template <int MODE, bool GATHER>
 __global__ __launch_bounds__(256) void k_planar_small(const float* __restrict__ x, float* y, const float* ysrc,
-                                                      const int16_t* __restrict__ idx, Geom g, int64_t total)
+                                                      const int16_t* __restrict__ idx, Geom g, int64_t total,
+                                                      const int32_t* __restrict__ owner)
 {
     const int RS = g.R * g.S;
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
@@ -984,7 +1025,9 @@ __global__ __launch_bounds__(256) void k_planar_small(const float* __restrict__ 
         if (GATHER) {
             y[st] = in ? x[pix] : 0.f;
         } else if (in) {
-            if (MODE == SCATTER_ASSIGN) y[pix] = x[st];
+            if (MODE == SCATTER_OWNED) {
+                if (owner[((int64_t)o.n * g.H + hh) * g.W + ww] == (int32_t)ib) y[pix] = x[st];
+            } else if (MODE == SCATTER_ASSIGN) y[pix] = x[st];
             else if (MODE == SCATTER_ADD) y[pix] = ysrc[pix] + x[st];
             else atomic_add_f32(y + pix, x[st]);
         }
@@ -1499,6 +1542,7 @@ static bool make_nhwc_args(const Geom& g, int numActive, int vec, NhwcArgs& a)
     a.units = (uint32_t)units;
     a.dCpb = make_fastdiv(a.cpb);
     a.dRow = make_fastdiv(a.rowV);
+    a.dCV = make_fastdiv((uint32_t)(g.C / vec));
     return true;
 }
 
@@ -1663,7 +1707,7 @@ static void gather_dispatch(const float* x, float* y, const int16_t* idx, const 
             const int64_t total = (int64_t)numActive * g.C * g.R * g.S;
             const int64_t wgs = (total + 255) / 256;
             hipLaunchKernelGGL((k_planar_small<SCATTER_ASSIGN, true>), dim3((unsigned)(wgs > 65536 ? 65536 : wgs)),
-                               dim3(256), 0, stream, x, y, (const float*)y, idx, g, total);
+                               dim3(256), 0, stream, x, y, (const float*)y, idx, g, total, (const int32_t*)nullptr);
             return;
         }
         hipLaunchKernelGGL(k_gather_planar<VEC>, tile_grid(a.grid2d, a.tpb, numActive, a.total), dim3(threads), lds,
@@ -1689,17 +1733,19 @@ hipError_t launch_gather(const float* x, float* y, const int16_t* idx, int numAc
 // "copy of the base + scatter" without copying the covered pixels first.
 template <int VEC, int MODE>
 static void scatter_dispatch(const float* x, float* y, const float* ysrc, const int16_t* idx, const Geom& g,
-                             int numActive, bool transpose, hipStream_t stream, hipError_t& err)
+                             int numActive, bool transpose, hipStream_t stream, hipError_t& err,
+                             const int32_t* owner = nullptr)
 {
+    const ColorArgs aux{1, 1, 0, nullptr, owner};
     if (!transpose) {
         NhwcArgs a;
         if (!make_nhwc_args(g, numActive, VEC, a)) { err = hipErrorInvalidValue; return; }
         if (nhwc_fits_buffers(g))
             hipLaunchKernelGGL((k_scatter_nhwc<VEC, MODE>), dim3((a.units + 3) / 4), dim3(256), 0, stream, x, y, ysrc,
-                               idx, a, ColorArgs{1, 1, 0, nullptr});
+                               idx, a, aux);
         else
             hipLaunchKernelGGL((k_scatter_nhwc_wide<VEC, MODE>), dim3((a.units + 3) / 4), dim3(256), 0, stream, x, y,
-                               ysrc, idx, a, ColorArgs{1, 1, 0, nullptr});
+                               ysrc, idx, a, aux);
     } else {
         TileArgs a;
         int threads;
@@ -1710,19 +1756,21 @@ static void scatter_dispatch(const float* x, float* y, const float* ysrc, const 
             const int64_t total = (int64_t)numActive * g.C * g.R * g.S;
             const int64_t wgs = (total + 255) / 256;
             hipLaunchKernelGGL((k_planar_small<MODE, false>), dim3((unsigned)(wgs > 65536 ? 65536 : wgs)), dim3(256),
-                               0, stream, x, y, ysrc, idx, g, total);
+                               0, stream, x, y, ysrc, idx, g, total, owner);
             return;
         }
         hipLaunchKernelGGL((k_scatter_planar<VEC, MODE>), tile_grid(a.grid2d, a.tpb, numActive, a.total), dim3(threads),
-                           lds, stream, x, y, ysrc, idx, a, ColorArgs{1, 1, 0, nullptr});
+                           lds, stream, x, y, ysrc, idx, a, aux);
     }
 }
 
 template <int VEC>
 static void scatter_mode(const float* x, float* y, const float* ysrc, const int16_t* idx, const Geom& g, int numActive,
-                         bool transpose, ScatterMode mode, hipStream_t stream, hipError_t& err)
+                         bool transpose, ScatterMode mode, hipStream_t stream, hipError_t& err, const int32_t* owner)
 {
-    if (mode == SCATTER_ASSIGN)
+    if (mode == SCATTER_ASSIGN && owner)
+        scatter_dispatch<VEC, SCATTER_OWNED>(x, y, ysrc, idx, g, numActive, transpose, stream, err, owner);
+    else if (mode == SCATTER_ASSIGN)
         scatter_dispatch<VEC, SCATTER_ASSIGN>(x, y, ysrc, idx, g, numActive, transpose, stream, err);
     else if (mode == SCATTER_ADD)
         scatter_dispatch<VEC, SCATTER_ADD>(x, y, ysrc, idx, g, numActive, transpose, stream, err);
@@ -1731,16 +1779,17 @@ static void scatter_mode(const float* x, float* y, const float* ysrc, const int1
 }
 
 static hipError_t scatter_from(const float* x, float* y, const float* ysrc, const int16_t* idx, int numActive,
-                               const Geom& g, bool transpose, ScatterMode mode, hipStream_t stream)
+                               const Geom& g, bool transpose, ScatterMode mode, hipStream_t stream,
+                               const int32_t* owner = nullptr)
 {
     if (numActive == 0) return hipSuccess;
     hipError_t err = hipSuccess;
     int vec = pick_vec(g, y, transpose ? nullptr : x);
     const int vsrc = pick_vec(g, ysrc, nullptr);
     if (vsrc < vec) vec = vsrc;
-    if (vec == 4) scatter_mode<4>(x, y, ysrc, idx, g, numActive, transpose, mode, stream, err);
-    else if (vec == 2) scatter_mode<2>(x, y, ysrc, idx, g, numActive, transpose, mode, stream, err);
-    else scatter_mode<1>(x, y, ysrc, idx, g, numActive, transpose, mode, stream, err);
+    if (vec == 4) scatter_mode<4>(x, y, ysrc, idx, g, numActive, transpose, mode, stream, err, owner);
+    else if (vec == 2) scatter_mode<2>(x, y, ysrc, idx, g, numActive, transpose, mode, stream, err, owner);
+    else scatter_mode<1>(x, y, ysrc, idx, g, numActive, transpose, mode, stream, err, owner);
     if (err != hipSuccess) return err;
     return hipGetLastError();
 }
@@ -1961,21 +2010,46 @@ __global__ __launch_bounds__(256) void k_cover_mark(const int16_t* __restrict__ 
     }
 }
 
-template <int VEC>
+// Owner map of the ordered plain scatter (SCATTER_OWNED): -1 everywhere, then the highest list position among the
+// blocks that cover each pixel.  Rows past the device-resident count and rows that name no image mark nothing.
+__global__ __launch_bounds__(256) void k_owner_fill(int32_t* __restrict__ owner, int64_t n)
+{
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) owner[i] = -1;
+}
+
+__global__ __launch_bounds__(256) void k_owner_mark(const int16_t* __restrict__ idx, int numActive, CoverArgs a,
+                                                    int32_t* __restrict__ owner)
+{
+    const int64_t total = (int64_t)numActive * a.RS;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const uint32_t ib = (uint32_t)(i / a.RS);
+        if (a.g.countDev && ib >= (uint32_t)*a.g.countDev) return;
+        const uint32_t p = (uint32_t)(i - (int64_t)ib * a.RS);
+        const uint32_t r = fdiv(p, a.dS), sc = p - r * (uint32_t)a.g.S;
+        const BlockOrigin o = load_origin(idx, ib, a.g);
+        const int hh = o.h0 + (int)r, ww = o.w0 + (int)sc;
+        if (o.valid && (unsigned)hh < (unsigned)a.g.H && (unsigned)ww < (unsigned)a.g.W)
+            atomicMax(owner + ((int64_t)o.n * a.imgPixels + (int64_t)hh * a.g.W + ww), (int32_t)ib);
+    }
+}
+
+// FLAG is the per-pixel coverage record: one byte (non-zero = covered), or the int32 owner map (>= 0 = covered).
+template <int VEC, typename FLAG>
 __global__ __launch_bounds__(256) void k_copy_uncovered(const float* __restrict__ src, float* __restrict__ dst,
-                                                        const uint8_t* __restrict__ flags, CoverArgs a)
+                                                        const FLAG* __restrict__ flags, CoverArgs a)
 {
     typedef typename Vec<VEC>::type vec;
     const uint32_t n = blockIdx.y;
     const rsrc_t sr = make_rsrc(src + (int64_t)n * a.imgFloats, a.imgBytes);
     const rsrc_t dr = make_rsrc(dst + (int64_t)n * a.imgFloats, a.imgBytes);
-    const uint8_t* __restrict__ fl = flags + (int64_t)n * a.imgPixels;
+    const FLAG* __restrict__ fl = flags + (int64_t)n * a.imgPixels;
     const uint32_t e0 = blockIdx.x * (256u * COVER_UNR) + threadIdx.x;
-    uint8_t cov[COVER_UNR];
+    bool cov[COVER_UNR];
 #pragma unroll
     for (int u = 0; u < COVER_UNR; ++u) {
         const uint32_t e = min(e0 + (uint32_t)u * 256u, a.imgV - 1u);
-        cov[u] = fl[fdiv(e, a.dCV)];
+        const FLAG f = fl[fdiv(e, a.dCV)];
+        cov[u] = sizeof(FLAG) == 1 ? f != 0 : (int32_t)f >= 0;
     }
     uint32_t off[COVER_UNR];
 #pragma unroll
@@ -1998,6 +2072,55 @@ size_t scatter_cover_workspace_bytes(const Geom& g, int numActive)
     return (((size_t)g.N * g.H * g.W + 3) & ~(size_t)3) + 16;
 }
 
+static void make_cover_args(const Geom& g, int vec, CoverArgs& c)
+{
+    c.g = g;
+    c.RS = (uint32_t)(g.R * g.S);
+    c.imgFloats = (int64_t)g.H * g.W * g.C;
+    c.imgPixels = (int64_t)g.H * g.W;
+    c.imgV = (uint32_t)(c.imgFloats / vec);
+    c.imgBytes = (uint32_t)(c.imgFloats * 4);
+    c.dCV = make_fastdiv((uint32_t)(g.C / vec));
+    c.dS = make_fastdiv((uint32_t)g.S);
+}
+
+size_t scatter_owner_workspace_bytes(const Geom& g, int numActive)
+{
+    if (numActive <= 0 || !(g.U < g.R || g.V < g.S)) return 0;  // only overlapping blocks need an order
+    if ((int64_t)g.R * g.S >= (1ll << 31)) return 0;
+    return (size_t)g.N * g.H * g.W * 4 + 16;
+}
+
+// Builds the owner map in `workspace`; false (nothing launched) when the ordered scatter does not apply.
+static bool build_owner_map(const int16_t* idx, int numActive, const Geom& g, void* workspace, size_t workspaceBytes,
+                            hipStream_t stream, int32_t*& owner)
+{
+    const size_t need = scatter_owner_workspace_bytes(g, numActive);
+    if (!workspace || need == 0 || workspaceBytes < need || (reinterpret_cast<uintptr_t>(workspace) & 3)) return false;
+    owner = static_cast<int32_t*>(workspace);
+    CoverArgs c;
+    make_cover_args(g, 1, c);
+    const int64_t n = (int64_t)g.N * g.H * g.W;
+    int64_t wgs = (n + 1023) / 1024;
+    if (wgs > 8192) wgs = 8192;
+    hipLaunchKernelGGL(k_owner_fill, dim3((unsigned)wgs), dim3(256), 0, stream, owner, n);
+    int64_t markWgs = ((int64_t)numActive * c.RS + 255) / 256;
+    if (markWgs > 65536) markWgs = 65536;
+    hipLaunchKernelGGL(k_owner_mark, dim3((unsigned)markWgs), dim3(256), 0, stream, idx, numActive, c, owner);
+    return true;
+}
+
+hipError_t launch_scatter_owned(const float* x, float* y, const int16_t* idx, int numActive, const Geom& g,
+                                bool transpose, void* workspace, size_t workspaceBytes, hipStream_t stream, bool& done)
+{
+    done = false;
+    if (numActive == 0) { done = true; return hipSuccess; }
+    int32_t* owner = nullptr;
+    if (!build_owner_map(idx, numActive, g, workspace, workspaceBytes, stream, owner)) return hipSuccess;
+    done = true;
+    return scatter_from(x, y, y, idx, numActive, g, transpose, SCATTER_ASSIGN, stream, owner);
+}
+
 hipError_t launch_scatter_over_base(const float* x, const float* ybase, float* y, const int16_t* idx, int numActive,
                                     const Geom& g, bool transpose, ScatterMode mode, void* workspace,
                                     size_t workspaceBytes, hipStream_t stream, bool& done)
@@ -2012,15 +2135,20 @@ hipError_t launch_scatter_over_base(const float* x, const float* ybase, float* y
     if ((int64_t)numActive * g.R * g.S * g.C * 4 < (16ll << 20)) return hipSuccess;
 
     CoverArgs c;
-    c.g = g;
-    c.RS = (uint32_t)(g.R * g.S);
     const int vec = pick_vec(g, ybase, y);
-    c.imgFloats = (int64_t)g.H * g.W * g.C;
-    c.imgPixels = (int64_t)g.H * g.W;
-    c.imgV = (uint32_t)(c.imgFloats / vec);
-    c.imgBytes = (uint32_t)(c.imgFloats * 4);
-    c.dCV = make_fastdiv((uint32_t)(g.C / vec));
-    c.dS = make_fastdiv((uint32_t)g.S);
+    make_cover_args(g, vec, c);
+    const dim3 grid((c.imgV + 256u * COVER_UNR - 1) / (256u * COVER_UNR), (unsigned)g.N);
+
+    // Plain writes of overlapping blocks: the owner map of the ordered scatter also tells which pixels are covered.
+    if (mode == SCATTER_ASSIGN && scatter_owner_workspace_bytes(g, numActive) != 0) {
+        int32_t* owner = nullptr;
+        if (!build_owner_map(idx, numActive, g, workspace, workspaceBytes, stream, owner)) return hipSuccess;
+        if (vec == 4) hipLaunchKernelGGL((k_copy_uncovered<4, int32_t>), grid, dim3(256), 0, stream, ybase, y, owner, c);
+        else if (vec == 2) hipLaunchKernelGGL((k_copy_uncovered<2, int32_t>), grid, dim3(256), 0, stream, ybase, y, owner, c);
+        else hipLaunchKernelGGL((k_copy_uncovered<1, int32_t>), grid, dim3(256), 0, stream, ybase, y, owner, c);
+        done = true;
+        return scatter_from(x, y, ybase, idx, numActive, g, transpose, mode, stream, owner);
+    }
     uint8_t* flags = static_cast<uint8_t*>(workspace);
 
     const int64_t words = (int64_t)((need - 16) / 4);
@@ -2030,10 +2158,10 @@ hipError_t launch_scatter_over_base(const float* x, const float* ybase, float* y
     int64_t markWgs = ((int64_t)numActive * c.RS + 255) / 256;
     if (markWgs > 65536) markWgs = 65536;
     hipLaunchKernelGGL(k_cover_mark, dim3((unsigned)markWgs), dim3(256), 0, stream, idx, numActive, c, flags);
-    const dim3 grid((c.imgV + 256u * COVER_UNR - 1) / (256u * COVER_UNR), (unsigned)g.N);
-    if (vec == 4) hipLaunchKernelGGL(k_copy_uncovered<4>, grid, dim3(256), 0, stream, ybase, y, flags, c);
-    else if (vec == 2) hipLaunchKernelGGL(k_copy_uncovered<2>, grid, dim3(256), 0, stream, ybase, y, flags, c);
-    else hipLaunchKernelGGL(k_copy_uncovered<1>, grid, dim3(256), 0, stream, ybase, y, flags, c);
+    const uint8_t* cflags = flags;
+    if (vec == 4) hipLaunchKernelGGL((k_copy_uncovered<4, uint8_t>), grid, dim3(256), 0, stream, ybase, y, cflags, c);
+    else if (vec == 2) hipLaunchKernelGGL((k_copy_uncovered<2, uint8_t>), grid, dim3(256), 0, stream, ybase, y, cflags, c);
+    else hipLaunchKernelGGL((k_copy_uncovered<1, uint8_t>), grid, dim3(256), 0, stream, ybase, y, cflags, c);
     done = true;
     return scatter_from(x, y, ybase, idx, numActive, g, transpose, mode, stream);
 }

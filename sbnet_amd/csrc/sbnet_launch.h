@@ -56,6 +56,14 @@ hipError_t launch_scatter_colored(const float* x, float* y, const int16_t* idx, 
                                   bool transpose, void* workspace, size_t workspaceBytes, hipStream_t stream,
                                   bool& done);
 
+// Plain writes ("=") of overlapping blocks in the order of the sequential CPU functor: on a pixel that several
+// blocks cover, the block listed last wins (sparse_gather.cc:105-129), for either stack layout and for lists that
+// name a block twice.  Needs scratch of scatter_owner_workspace_bytes() (one int32 per pixel; 0 when the blocks do
+// not overlap and no order is needed); `done` is false when that is missing and nothing was launched.
+size_t scatter_owner_workspace_bytes(const Geom& g, int numActive);
+hipError_t launch_scatter_owned(const float* x, float* y, const int16_t* idx, int numActive, const Geom& g,
+                                bool transpose, void* workspace, size_t workspaceBytes, hipStream_t stream, bool& done);
+
 // y = copy of ybase with the blocks written ("=") or added ("+=", non-overlapping) on top, moving every byte once:
 // pixels that no active block covers are copied, covered ones are written by the scatter kernels, which read
 // ybase where they add.  Needs scratch of scatter_cover_workspace_bytes() for one flag byte per pixel; `done` is

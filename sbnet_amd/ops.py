@@ -60,7 +60,23 @@ def _dev_f32(t, name):
 def _idx_i16(t):
     if not isinstance(t, torch.Tensor) or not t.is_cuda or t.dtype != torch.int16:
         raise TypeError("active_block_indices must be an int16 tensor on the GPU")
+    if t.dim() != 2 or t.shape[1] != 3:
+        raise InvalidArgument("active_block_indices must have shape [blocks, 3], got %s" % (tuple(t.shape),))
     return t.contiguous()
+
+
+def _check_count(M, idx):
+    """The kernels read M rows of the list: a count beyond it would read past the allocation (the reference does
+    not check this either, sparse_gather.cc:190-192; here it is an error instead of a device fault)."""
+    if M < 0 or M > int(idx.shape[0]):
+        raise InvalidArgument("bin_counts[0] = %d is outside the block list of %d rows" % (M, int(idx.shape[0])))
+
+
+def _check_stack(t, M, C, R, S, transpose, name):
+    want = (C, R, S) if transpose else (R, S, C)
+    if t.dim() != 4 or tuple(int(d) for d in t.shape[1:]) != want or int(t.shape[0]) < M:
+        raise InvalidArgument("%s must be a block stack of shape [>=%d, %s], got %s" %
+                              (name, M, ", ".join(str(d) for d in want), tuple(t.shape)))
 
 
 def _count(bin_counts):
@@ -107,8 +123,8 @@ def reduce_mask(mask, dynamic_bcount, dynamic_bsize, dynamic_bstride, dynamic_bo
     """
     lib = _lib.load()
     mask = _dev_f32(mask, "mask")
-    if mask.dim() < 3:
-        raise InvalidArgument("mask must be [N,H,W,1]")
+    if mask.dim() not in (3, 4) or (mask.dim() == 4 and mask.shape[3] != 1):
+        raise InvalidArgument("mask must be [N,H,W,1] (or [N,H,W]), got %s" % (tuple(mask.shape),))
     N, H, W = int(mask.shape[0]), int(mask.shape[1]), int(mask.shape[2])
     bc, bcp, bcl = _pair(dynamic_bcount)
     bs, bsp, bsl = _pair(dynamic_bsize)
@@ -160,10 +176,17 @@ def gather_forward(x, bin_counts, active_block_indices, dynamic_bsize, dynamic_b
     dims, rank = _dims(x)
     y = out
     with torch.cuda.device(x.device):
-        if y is None and rank == 4 and bsl == 2:
+        if rank == 4 and bsl == 2 and btl == 2 and bol == 2:
+            # past the checks the library reports in the reference's order: sizes the kernels rely on
+            _check_count(M, idx)
             C, R, S = int(x.shape[3]), int(bs[0]), int(bs[1])
-            shape = (M, C, R, S) if transpose else (M, R, S, C)
-            y = torch.empty(shape, dtype=torch.float32, device=x.device)
+            if y is None:
+                y = torch.empty((M, C, R, S) if transpose else (M, R, S, C), dtype=torch.float32, device=x.device)
+            else:
+                if not isinstance(y, torch.Tensor) or y.device != x.device or y.dtype != torch.float32 or \
+                        not y.is_contiguous():
+                    raise TypeError("out must be a contiguous float32 tensor on the device of x")
+                _check_stack(y, M, C, R, S, transpose, "out")
         yp = y.data_ptr() if y is not None else None
         if dcount is not None:
             _check(lib.sbnet_sparse_gather_device_count(x.data_ptr(), dims, rank, dcount.data_ptr(), M, idx.data_ptr(),
@@ -192,11 +215,16 @@ def scatter_forward(x, bin_counts, active_block_indices, ybase, dynamic_bsize, d
     bt, btp, btl = _pair(dynamic_bstride)
     bo, bop, bol = _pair(dynamic_boffset)
     dims, rank = _dims(ybase)
+    overlap = bsl == 2 and btl == 2 and (bt[0] < bs[0] or bt[1] < bs[1])
+    if rank == 4 and bsl == 2 and btl == 2 and bol == 2 and (atomic or not add or not overlap):
+        _check_count(M, idx)
+        _check_stack(x, M, int(ybase.shape[3]), int(bs[0]), int(bs[1]), transpose, "x")
     with torch.cuda.device(ybase.device):
         ws_ptr, ws_bytes = None, 0
-        if (add and atomic) or not use_var:
-            # scratch for the atomic-free scatter-add of overlapping blocks, and for building the copying op's
-            # output in one pass (uncovered pixels copied, covered ones scattered)
+        if (add and atomic) or not use_var or (not add and overlap):
+            # scratch for the atomic-free scatter-add of overlapping blocks, for overlapping plain writes in the
+            # CPU functor's order (the block listed last wins), and for building the copying op's output in one
+            # pass (uncovered pixels copied, covered ones scattered)
             need = lib.sbnet_sparse_scatter_workspace_bytes(M, dims, rank, bsp, bsl, btp, btl, bop, bol)
             if need:
                 ws = _workspace(ybase.device, need)

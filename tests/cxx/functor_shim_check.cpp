@@ -23,11 +23,12 @@ template <typename Device, typename T> struct SparseScatterFunctor {
 };
 template <typename Device, typename T> struct CopyTensorFunctor {
     void operator()(const Device& d, T* dst, const T* src, int count);
+    void** getStream(const Device& d);
 };
 
 struct FakeGpuDevice {
     void* s;
-    void* stream() const { return s; }
+    void* const& stream() const { return s; }  // a reference, as Eigen::GpuDevice::stream() returns
 };
 
 #include "sbnet_reference_functors.hpp"
@@ -61,6 +62,13 @@ int main()
     SparseGatherFunctor<FakeGpuDevice, float>()(d, nof, 1, 8, 8, 4, nullptr, 0, 0, 2, 2, 2, 2, 0, nullptr, false);
     CopyTensorFunctor<FakeGpuDevice, float>()(d, nullptr, nof, 0);
     if (g_calls != 4) return 5;
+    // getStream hands out the address of the device's stream handle (sparse_gather.cu:275)
+    if (CopyTensorFunctor<FakeGpuDevice, float>().getStream(d) != &d.s) return 6;
+    // a scratch provider of the caller's replaces the library's
+    sbnet_amd::scratch_provider() = [](size_t, void*) -> void* { ++g_calls; return nullptr; };
+    SparseScatterFunctor<FakeGpuDevice, float>()(d, nof, 1, 8, 8, 4, nullptr, 0, 0, 2, 2, 2, 2, 3, nullptr, true, false,
+                                                 true);
+    if (g_calls != 6 || g_last != SBNET_EINVAL_ARG) return 7;  // one call of the provider, one of the handler
     std::printf("functor shim ok\n");
     return 0;
 }

@@ -37,6 +37,8 @@ MASK_8x8 = [[0, 0, 0, 0, 0, 1, 1, 1],
 # mask -> gather -> VALID conv with an all-ones kernel on an all-ones input -> scatter (add=False)
 # into a zero tensor of the output size.  y_exp counts the in-image pixels of each kernel window on
 # active blocks (4 / 6 / 9 at corners / edges / interior for 3x3) and is 0 where no block is active.
+# The scatter steps by `s_bstride` output pixels where given, else by `bstride` (equal to bsize_out for a
+# convolution of stride 1).
 PIPELINE = [
     dict(name="mask_valid_3x3", source="benchmark/sparse_conv_tests.py:197-218",
          mask=MASK_5x5, bsize=[3, 3], ksize=[3, 3], conv_strides=[1, 1], padding="VALID",
@@ -50,6 +52,13 @@ PIPELINE = [
          mask=MASK_5x5, bsize=[4, 4], ksize=[3, 3], conv_strides=[1, 1], padding="SAME",
          bstride=[2, 2], boffset=[-1, -1], bcount=[3, 3], bsize_out=[2, 2],
          y_exp=[[4, 6, 6, 6, 0], [6, 9, 9, 9, 0], [6, 9, 9, 9, 0], [6, 9, 9, 9, 0], [0, 0, 0, 0, 0]]),
+    # the only table whose convolution has a stride: gather blocks step by bsize - k + stride = 4 input pixels,
+    # the 2x2 outputs of a block step by 4 / 2 = 2 output pixels (`s_bstride`); one block at offset -1 covers
+    # the whole 5x5 input, and the 3x3 output shows its four windows with 2x2, 2x3, 3x2 and 3x3 in-image pixels
+    dict(name="mask_same_even_block_strides_5x5_s2", source="benchmark/sparse_conv_tests.py:270-291",
+         mask=MASK_5x5, bsize=[5, 5], ksize=[3, 3], conv_strides=[2, 2], padding="SAME",
+         bstride=[4, 4], boffset=[-1, -1], bcount=[1, 1], bsize_out=[2, 2], s_bstride=[2, 2],
+         y_exp=[[4, 6, 0], [6, 9, 0], [0, 0, 0]]),
     dict(name="mask_valid_large_block_5x5_k2", source="benchmark/sparse_conv_tests.py:293-321",
          mask=MASK_8x8, bsize=[5, 5], ksize=[2, 2], conv_strides=[1, 1], padding="VALID",
          bstride=[4, 4], boffset=[0, 0], bcount=[2, 2], bsize_out=[4, 4],

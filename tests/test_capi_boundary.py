@@ -56,20 +56,24 @@ def test_scatter_workspace_query():
     lib = _lib.load()
     dims = I64x4(2, 512, 512, 256)
     flags = 2 * 512 * 512 + 16   # one flag byte per pixel: the copying scatter built in one pass
-    # 16x16 blocks at stride 8: 2x2 blocks cover a pixel, the atomic-free method applies
-    n = lib.sbnet_sparse_scatter_workspace_bytes(2000, dims, 4, I32x2(16, 16), 2, I32x2(8, 8), 2, I32x2(0, 0), 2)
-    assert n >= max(2 * 64 * 64 * 4 + 2000 * 4, flags)
-    # 16x16 at stride 4: 4x4 blocks cover a pixel: the add runs in 16 passes, which needs the block map only
-    # (less than the flag bytes here)
-    n = lib.sbnet_sparse_scatter_workspace_bytes(2000, dims, 4, I32x2(16, 16), 2, I32x2(4, 4), 2, I32x2(0, 0), 2)
-    assert n == max(flags, n) and 2 * 128 * 128 * 4 <= n < max(2 * 140 * 140 * 4, flags + 1)
-    # 16x16 at stride 3: 6x6 blocks cover a pixel, beyond both atomic-free methods: the flag bytes only
-    assert lib.sbnet_sparse_scatter_workspace_bytes(2000, dims, 4, I32x2(16, 16), 2, I32x2(3, 3), 2, I32x2(0, 0),
+    owner = 2 * 512 * 512 * 4 + 16  # one int32 per pixel: overlapping plain writes in the CPU functor's order
+    # blocks that tile (stride == size): no order is needed, only the flag bytes
+    assert lib.sbnet_sparse_scatter_workspace_bytes(2000, dims, 4, I32x2(16, 16), 2, I32x2(16, 16), 2, I32x2(0, 0),
                                                     2) == flags
-    # an image of 2^30 floats or more is beyond the one-pass copy as well
+    # 16x16 blocks at stride 8: 2x2 blocks cover a pixel, the atomic-free add applies
+    n = lib.sbnet_sparse_scatter_workspace_bytes(2000, dims, 4, I32x2(16, 16), 2, I32x2(8, 8), 2, I32x2(0, 0), 2)
+    assert n >= max(2 * 64 * 64 * 4 + 2000 * 4, owner)
+    # 16x16 at stride 4: 4x4 blocks cover a pixel: the add runs in 16 passes, which needs the block map only
+    # (less than the owner map here)
+    n = lib.sbnet_sparse_scatter_workspace_bytes(2000, dims, 4, I32x2(16, 16), 2, I32x2(4, 4), 2, I32x2(0, 0), 2)
+    assert n == owner
+    # 16x16 at stride 3: 6x6 blocks cover a pixel, beyond both atomic-free adds: the owner map only
+    assert lib.sbnet_sparse_scatter_workspace_bytes(2000, dims, 4, I32x2(16, 16), 2, I32x2(3, 3), 2, I32x2(0, 0),
+                                                    2) == owner
+    # an image of 2^30 floats or more is beyond the one-pass copy; the owner map still applies to it
     big = I64x4(1, 32768, 32768, 1)
     assert lib.sbnet_sparse_scatter_workspace_bytes(2000, big, 4, I32x2(16, 16), 2, I32x2(3, 3), 2, I32x2(0, 0),
-                                                    2) == 0
+                                                    2) == 32768 * 32768 * 4 + 16
     assert lib.sbnet_sparse_scatter_workspace_bytes(2000, dims, 3, I32x2(16, 16), 2, I32x2(8, 8), 2, I32x2(0, 0),
                                                     2) == 0
 
@@ -159,6 +163,29 @@ def test_reference_functor_header_compiles_links_and_reports_errors():
     exe = os.path.join(ROOT, "tests", "cxx", "_build", "functor_shim_check")
     out = subprocess.run([exe], check=True, capture_output=True, text=True)
     assert "functor shim ok" in out.stdout
+
+
+def test_python_mirror_checks_sizes_before_any_launch():
+    """The kernels trust the count, the list and the stack shapes: the Python mirror refuses what would make them
+    read or write past an allocation (the reference's ops do not check these, sparse_gather.cc:190-192, 332)."""
+    import torch
+    from sbnet_amd import ops
+
+    idx = torch.zeros((5, 3), dtype=torch.int16)
+    ops._check_count(0, idx)
+    ops._check_count(5, idx)
+    for bad in (-1, 6):
+        with pytest.raises(ops.InvalidArgument, match="outside the block list"):
+            ops._check_count(bad, idx)
+    ops._check_stack(torch.zeros((5, 3, 4, 8)), 5, 8, 3, 4, False, "x")
+    ops._check_stack(torch.zeros((7, 8, 3, 4)), 5, 8, 3, 4, True, "x")
+    for shape, transpose in (((4, 3, 4, 8), False),      # fewer blocks than the count
+                             ((5, 8, 3, 4), False),      # planar stack given as NHWC
+                             ((5, 3, 4, 8), True),       # and the other way round
+                             ((5, 3, 4, 7), False),      # channel count of another tensor
+                             ((5, 3, 4), False)):        # not rank 4
+        with pytest.raises(ops.InvalidArgument, match="block stack of shape"):
+            ops._check_stack(torch.zeros(shape), 5, 8, 3, 4, transpose, "x")
 
 
 def test_python_mirror_fails_loudly_without_library(monkeypatch):

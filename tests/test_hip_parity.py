@@ -146,13 +146,14 @@ def test_pipeline_known_answers(case, transpose, use_var):
     p = sbnet_amd.sparse_gather(dev(x), r.bin_counts, r.active_block_indices, case["bsize"], case["bstride"],
                                 case["boffset"], transpose=transpose)
     p = host(p)
-    q = box_sum_valid(p.transpose(0, 2, 3, 1) if transpose else p, case["ksize"][0], case["ksize"][1])
+    q = box_sum_valid(p.transpose(0, 2, 3, 1) if transpose else p, case["ksize"][0], case["ksize"][1],
+                      *case["conv_strides"])
     if transpose:
         q = np.ascontiguousarray(q.transpose(0, 3, 1, 2))
     y_exp = np.asarray(case["y_exp"], np.float32)[None, :, :, None]
     fn = sbnet_amd.sparse_scatter_var if use_var else sbnet_amd.sparse_scatter
     y = fn(dev(q), r.bin_counts, r.active_block_indices, dev(np.zeros_like(y_exp)), case["bsize_out"],
-           case["bstride"], [0, 0], add=False, transpose=transpose)
+           case.get("s_bstride", case["bstride"]), [0, 0], add=False, transpose=transpose)
     np.testing.assert_array_equal(host(y), y_exp)
 
 
@@ -652,6 +653,95 @@ def test_overlapping_add_is_exact_and_ordered(geom):
     np.testing.assert_array_equal(host(bd), y_o)
 
 
+@pytest.mark.parametrize("geom", [
+    # (N, H, W, C), bsize, bstride, boffset
+    ((2, 40, 52, 8), (6, 6), (3, 3), (-2, -1)),          # 2x2 blocks per pixel
+    ((1, 33, 47, 5), (5, 7), (3, 4), (-2, -3)),          # scalar channel vectors
+    ((1, 30, 30, 6), (7, 7), (2, 2), (0, 0)),            # 4x4 blocks per pixel
+    ((1, 64, 64, 16), (10, 10), (8, 8), (-1, -1)),       # the plumbing configuration's geometry
+    ((1, 120, 130, 32), (27, 27), (25, 25), (-1, -1)),   # planes split over tiles
+    ((2, 64, 72, 256), (16, 16), (8, 8), (0, 0)),        # the atomic scatter-add configuration's geometry
+    ((3, 20, 20, 4), (1, 3), (1, 2), (0, 0)),            # planes below 4 pixels (generic planar kernel)
+])
+def test_overlapping_plain_writes_follow_list_order(geom):
+    """add=False on overlapping blocks that carry different values: the sequential CPU functor lets the block
+    listed last win on every shared pixel (sparse_gather.cc:105-129).  Shuffled lists, a block listed twice,
+    both stack layouts, the in-place and the copying op, host and device count."""
+    (N, H, W, C), bs, bst, bo = geom
+    rng = np.random.default_rng(H * 7 + C)
+    bc = bcount_covering(H, W, bst, bo)
+    cells = [(n, i, j) for n in range(N) for i in range(bc[0]) for j in range(bc[1]) if rng.random() < 0.7]
+    idx = np.array(cells + cells[:3], np.int16)   # three blocks appear twice, with different stack rows
+    rng.shuffle(idx, axis=0)
+    M = len(idx)
+    cnt = np.array([M], np.int32)
+    base = rng.standard_normal((N, H, W, C)).astype(np.float32)
+    idxd = dev(idx)
+    dcount = torch.tensor([M - 2], dtype=torch.int32, device=DEV)
+    for transpose in (False, True):
+        shape = (M, C, bs[0], bs[1]) if transpose else (M, bs[0], bs[1], C)
+        stack = rng.standard_normal(shape).astype(np.float32)
+        y_o = orc.sparse_scatter(stack, cnt, idx, base, bs, bst, bo, add=False, transpose=transpose)
+        assert not np.array_equal(y_o, orc.sparse_scatter(stack[::-1].copy(), cnt, idx[::-1].copy(), base, bs, bst, bo,
+                                                          add=False, transpose=transpose)), "order must matter here"
+        sd = dev(stack)
+        y = sbnet_amd.sparse_scatter(sd, cnt, idxd, dev(base), bs, bst, bo, add=False, transpose=transpose)
+        np.testing.assert_array_equal(host(y), y_o)
+        yv = dev(base)
+        sbnet_amd.sparse_scatter_var(sd, cnt, idxd, yv, bs, bst, bo, add=False, transpose=transpose)
+        np.testing.assert_array_equal(host(yv), y_o)
+        # the count on the device: the last two rows of the list do not take part
+        y_o2 = orc.sparse_scatter(stack, [M - 2], idx, base, bs, bst, bo, add=False, transpose=transpose)
+        yv = dev(base)
+        sbnet_amd.sparse_scatter_var(sd, dcount, idxd, yv, bs, bst, bo, add=False, transpose=transpose)
+        np.testing.assert_array_equal(host(yv), y_o2)
+        y = sbnet_amd.sparse_scatter(sd, dcount, idxd, dev(base), bs, bst, bo, add=False, transpose=transpose)
+        np.testing.assert_array_equal(host(y), y_o2)
+
+
+def test_overlapping_plain_writes_large_enough_for_the_one_pass_copy():
+    """The copying op on 16 MB or more of blocks builds its output from uncovered pixels (copied) and covered
+    ones (scattered); with overlapping plain writes both parts are told apart by the owner map."""
+    rng = np.random.default_rng(5)
+    N, H, W, C = 1, 256, 256, 64
+    bs, bst, bo = (18, 18), (16, 16), (-1, -1)
+    bc = bcount_covering(H, W, bst, bo)
+    cells = [(0, i, j) for i in range(bc[0]) for j in range(bc[1]) if rng.random() < 0.8]
+    idx = np.array(cells, np.int16)
+    rng.shuffle(idx, axis=0)
+    M = len(idx)
+    assert M * bs[0] * bs[1] * C * 4 >= (16 << 20)
+    base = rng.standard_normal((N, H, W, C)).astype(np.float32)
+    for transpose in (False, True):
+        shape = (M, C, bs[0], bs[1]) if transpose else (M, bs[0], bs[1], C)
+        stack = rng.standard_normal(shape).astype(np.float32)
+        y_o = orc.sparse_scatter(stack, [M], idx, base, bs, bst, bo, add=False, transpose=transpose)
+        y = sbnet_amd.sparse_scatter(dev(stack), [M], dev(idx), dev(base), bs, bst, bo, add=False, transpose=transpose)
+        np.testing.assert_array_equal(host(y), y_o)
+
+
+@pytest.mark.parametrize("geom", [((63, 63), 32), ((65, 65), 32), ((31, 31), 33), ((127, 127), 16), ((63, 63), 18)])
+def test_planar_scatter_short_last_split(geom):
+    """Block planes whose split into tiles leaves 1-3 pixels for the last tile (63x63 = 31*128 + 1 pixels with
+    32 channels): the transposed scatter moves that tail float by float; every mode against the oracle."""
+    (R, S), C = geom
+    rng = np.random.default_rng(R * S + C)
+    N, H, W = 1, R + 9, 2 * S + 5
+    bs, bst, bo = (R, S), (R, S), (-3, -2)
+    idx = np.array([(0, 0, 0), (0, 0, 1), (0, 1, 0), (0, 1, 2)], np.int16)
+    M = len(idx)
+    stack = rng.integers(-8, 9, size=(M, C, R, S)).astype(np.float32)
+    base = rng.integers(-4, 5, size=(N, H, W, C)).astype(np.float32)
+    g_o = orc.sparse_gather(base, [M], idx, bs, bst, bo, transpose=True)
+    g = sbnet_amd.sparse_gather(dev(base), [M], dev(idx), bs, bst, bo, transpose=True)
+    np.testing.assert_array_equal(host(g), g_o)
+    for add, atomic in ((False, False), (True, False), (True, True)):
+        y_o = orc.sparse_scatter(stack, [M], idx, base, bs, bst, bo, add=add, atomic=atomic, transpose=True)
+        yv = dev(base)
+        sbnet_amd.sparse_scatter_var(dev(stack), [M], dev(idx), yv, bs, bst, bo, add=add, atomic=atomic, transpose=True)
+        np.testing.assert_array_equal(host(yv), y_o, err_msg="add %s atomic %s" % (add, atomic))
+
+
 def test_overlapping_add_with_repeated_blocks_falls_back_to_atomics():
     rng = np.random.default_rng(77)
     N, H, W, C = 1, 24, 24, 8
@@ -782,8 +872,6 @@ def test_device_resident_count(geom):
         g[M:] = 1.0e6
         base = rng.integers(-4, 5, size=(N, H, W, C)).astype(np.float32)
         for add, atomic in ((False, False), (True, True)) if overlap else ((False, False), (True, False), (True, True)):
-            if not add and overlap:
-                continue  # overlapping plain writes of different blocks race on the GPU
             y_o = orc.sparse_scatter(g_o, cnt_o, idx_o, base, bs, bst, bo, add=add, atomic=atomic,
                                      transpose=transpose)
             y = sbnet_amd.sparse_scatter(g, r.bin_counts, r.active_block_indices, dev(base), bs, bst, bo, add=add,
@@ -877,7 +965,8 @@ def test_random_geometries(seed):
             np.testing.assert_array_equal(host(g), g_o, err_msg=tag)
             stack = rng.integers(-8, 9, size=g_o.shape).astype(np.float32)
             sd = dev(stack)
-            modes = [(True, True)] if overlap else [(False, False), (True, False), (True, True)]
+            # (plain writes of overlapping blocks with different values: the block listed last wins)
+            modes = [(False, False), (True, True)] if overlap else [(False, False), (True, False), (True, True)]
             for add, atomic in modes:
                 y_o = orc.sparse_scatter(stack, cnt, idx, base, bs, bst, bo, add=add, atomic=atomic,
                                          transpose=transpose)

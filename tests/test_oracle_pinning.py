@@ -59,13 +59,13 @@ def test_pipeline_known_answers(case, transpose):
     idx, cnt = orc.reduce_mask(mask, case["bcount"], case["bsize"], case["bstride"], case["boffset"], 0.0)
     p = orc.sparse_gather(x, cnt, idx, case["bsize"], case["bstride"], case["boffset"], transpose=transpose)
     p_nhwc = p.transpose(0, 2, 3, 1) if transpose else p
-    q = box_sum_valid(p_nhwc, case["ksize"][0], case["ksize"][1])
+    q = box_sum_valid(p_nhwc, case["ksize"][0], case["ksize"][1], *case["conv_strides"])
     assert list(q.shape[1:3]) == case["bsize_out"]
     if transpose:
         q = np.ascontiguousarray(q.transpose(0, 3, 1, 2))
     y_exp = np.asarray(case["y_exp"], np.float32)[None, :, :, None]
-    y = orc.sparse_scatter(q, cnt, idx, np.zeros_like(y_exp), case["bsize_out"], case["bstride"], [0, 0],
-                           add=False, transpose=transpose)
+    y = orc.sparse_scatter(q, cnt, idx, np.zeros_like(y_exp), case["bsize_out"], case.get("s_bstride", case["bstride"]),
+                           [0, 0], add=False, transpose=transpose)
     np.testing.assert_array_equal(y, y_exp)
 
 

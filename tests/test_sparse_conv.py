@@ -34,7 +34,8 @@ def covered(indices, bp, shape):
 
 @pytest.mark.parametrize("transpose", [False, True])
 @pytest.mark.parametrize("use_var", [False, True])
-@pytest.mark.parametrize("case", [c for c in GOLD["pipeline"] if c["padding"] == "SAME"], ids=lambda c: c["name"])
+@pytest.mark.parametrize("case", [c for c in GOLD["pipeline"] if c["padding"] == "SAME" and
+                                  c["conv_strides"] == [1, 1]], ids=lambda c: c["name"])
 def test_sparse_conv2d_custom_known_answers(case, use_var, transpose):
     """SparseConv2DCustomTests._test_sparse_conv2d_custom_with_mask (sparse_conv_tests.py:400-435): the expected
     output is y_exp with the input (ones) showing through wherever no block wrote."""
