@@ -212,12 +212,8 @@ int reduce_mask_impl(const float* mask, int N, int H, int W, const int32_t* bcou
     bool haveCount = false;
     if (e == hipSuccess && sig) haveCount = poll_host_signal(*sig, seq, stream, countHost, &e);
     if (e == hipSuccess && countHost && !haveCount) {
-        // the count sits in countDev, or behind the flags and counts of the workspace
-        const int32_t* src = countDev;
-        if (!src) {
-            const size_t flagBytes = ((size_t)T + 15) & ~(size_t)15;
-            src = reinterpret_cast<const int32_t*>(static_cast<const uint8_t*>(ws) + flagBytes) + T;
-        }
+        // the count sits in countDev, or in the workspace
+        const int32_t* src = countDev ? countDev : sbnet::reduce_mask_count_slot(ws, T);
         e = hipMemcpyAsync(countHost, src, sizeof(int32_t), hipMemcpyDeviceToHost, stream);
         if (e == hipSuccess) e = hipStreamSynchronize(stream);
     }

@@ -23,9 +23,11 @@ struct Geom {
 
 enum ScatterMode { SCATTER_ASSIGN = 0, SCATTER_ADD = 1, SCATTER_ATOMIC = 2 };
 
-// reduce_mask scratch layout: one flag byte per sparsity block, then one int32 count per
-// pooling workgroup, then one int32 for the total when the caller gives no device count.
+// reduce_mask scratch: words of the one-launch mode, one flag byte per sparsity block, one int32 count per
+// pooling workgroup, one int32 for the total when the caller gives no device count.  Its contents before a
+// call do not matter.  reduce_mask_count_slot: where the total goes when the caller gives no device count.
 size_t reduce_mask_workspace_bytes(int64_t totalBlocks);
+int32_t* reduce_mask_count_slot(void* workspace, int64_t totalBlocks);
 
 // hostSignal (optional): device-visible address of an 8-byte word in pinned host memory; the kernel that knows
 // the count stores (hostSeq << 32 | count) there, so a host that polls the word needs no copy and no stream
