@@ -50,7 +50,9 @@ typedef enum sbnet_status {
        a workspace that is too small, y aliasing ybase in the copying scatter. */
     SBNET_EINVAL_ARG = 4,
     /* A HIP runtime call failed; sbnet_last_hip_error() has the hipError_t. */
-    SBNET_EHIP = 5
+    SBNET_EHIP = 5,
+    /* sbnet_reduce_mask_static: the problem needs more scratch than the library's own array holds. */
+    SBNET_ETOOBIG = 6
 } sbnet_status;
 
 /* Human-readable text for a status; the InvalidArgument texts are the reference's. */
@@ -111,6 +113,30 @@ int sbnet_reduce_mask(const float* mask, int N, int H, int W,
                       int16_t* active_block_indices,
                       int32_t* bin_counts_host, int32_t* bin_counts_device,
                       void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * sbnet_reduce_mask for callers that cannot allocate and have no workspace to bring: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  The
+ * scratch is an array inside the library's code object (2 MiB per GPU, held until the process ends); the call
+ * allocates nothing, on the device or the host, and frees nothing.  For the same reason the count goes to
+ * bin_counts_device only (required): the host-visible count of sbnet_reduce_mask needs a word of pinned host
+ * memory.  Everything else (arguments, checks, order of the list, zero-count fix-up, asynchronous on `stream`)
+ * is sbnet_reduce_mask's.
+ *   Limit: N * bcount[0] * bcount[1] <= sbnet_reduce_mask_static_max_indices() (about 400 000 blocks);
+ *   beyond that the call returns SBNET_ETOOBIG and launches nothing.
+ *   Every call on a GPU uses that GPU's one array: calls that may run at the same time on one GPU (different
+ *   streams, different threads) race on it and must be serialised by the caller; calls on one stream are.
+ *   Nothing in the array has to be cleared between calls (the kernel tells a call's data from what an earlier
+ *   call left by a per-call tag), so a smaller problem may follow a larger one.
+ */
+int sbnet_reduce_mask_static(const float* mask, int N, int H, int W,
+                             const int32_t* bcount, int bcount_len,
+                             const int32_t* bsize, int bsize_len,
+                             const int32_t* bstride, int bstride_len,
+                             const int32_t* boffset, int boffset_len,
+                             float tol, int avgpool,
+                             int16_t* active_block_indices, int32_t* bin_counts_device, void* stream);
+int64_t sbnet_reduce_mask_static_max_indices(void);
 
 /*
  * Functor level: replaces ReduceMaskFunctor<GPUDevice,float>::operator()

@@ -16,6 +16,7 @@ SBNET_EINVAL_RANK = 2
 SBNET_EINVAL_OVERLAP = 3
 SBNET_EINVAL_ARG = 4
 SBNET_EHIP = 5
+SBNET_ETOOBIG = 6
 
 _vp = ctypes.c_void_p
 _int = ctypes.c_int
@@ -35,6 +36,9 @@ SIGNATURES = {
     "sbnet_reduce_mask_workspace_bytes": (_sz, [_int, _i32p, _int]),
     "sbnet_reduce_mask": (_int, [_vp, _int, _int, _int, _i32p, _int, _i32p, _int, _i32p, _int, _i32p, _int,
                                  _f, _int, _vp, _i32p, _vp, _vp, _sz, _vp]),
+    "sbnet_reduce_mask_static": (_int, [_vp, _int, _int, _int, _i32p, _int, _i32p, _int, _i32p, _int, _i32p, _int,
+                                        _f, _int, _vp, _vp, _vp]),
+    "sbnet_reduce_mask_static_max_indices": (ctypes.c_int64, []),
     "sbnet_reduce_mask_functor": (_int, [_vp, _int, _int, _int, _f] + [_int] * 8 + [_uint, _uint, _vp, _vp, _int,
                                                                                      _vp, _sz, _vp]),
     "sbnet_sparse_gather": (_int, [_vp, _i64p, _int, _i32, _vp, _i32p, _int, _i32p, _int, _i32p, _int, _int,

@@ -306,6 +306,9 @@ const char* sbnet_status_string(int status)
         return "InvalidArgument: Only non-overlapping blocks are supported with add=True, atomic=False";
     case SBNET_EINVAL_ARG: return "InvalidArgument: null pointer, size out of range or workspace too small";
     case SBNET_EHIP: return "HIP runtime error (see sbnet_last_hip_error)";
+    case SBNET_ETOOBIG:
+        return "InvalidArgument: more blocks than the library's own scratch holds (sbnet_reduce_mask_static_max_indices); "
+               "use sbnet_reduce_mask with a workspace";
     default: return "unknown sbnet status";
     }
 }
@@ -335,6 +338,37 @@ int sbnet_reduce_mask(const float* mask, int N, int H, int W, const int32_t* bco
     return reduce_mask_impl(mask, N, H, W, bcount, bsize, bstride, boffset, tol, avgpool, true,
                             active_block_indices, bin_counts_host, bin_counts_device, workspace,
                             workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+int sbnet_reduce_mask_static(const float* mask, int N, int H, int W, const int32_t* bcount, int bcount_len,
+                             const int32_t* bsize, int bsize_len, const int32_t* bstride, int bstride_len,
+                             const int32_t* boffset, int boffset_len, float tol, int avgpool,
+                             int16_t* active_block_indices, int32_t* bin_counts_device, void* stream)
+{
+    if (!pair_ok(bcount, bcount_len) || !pair_ok(bsize, bsize_len) || !pair_ok(bstride, bstride_len) ||
+        !pair_ok(boffset, boffset_len))
+        return SBNET_EINVAL_PARAM_SHAPE;
+    if (!bin_counts_device) return SBNET_EINVAL_ARG;
+    const int64_t T = sbnet_reduce_mask_max_indices(N, bcount, bcount_len);
+    if (T < 0 || T >= (1ll << 31) || sbnet::reduce_mask_workspace_bytes(T) > sbnet::STATIC_SCRATCH_BYTES)
+        return SBNET_ETOOBIG;
+    void* ws = nullptr;
+    SBNET_HIP(sbnet::static_scratch(&ws));
+    return reduce_mask_impl(mask, N, H, W, bcount, bsize, bstride, boffset, tol, avgpool, true, active_block_indices,
+                            nullptr, bin_counts_device, ws, sbnet::STATIC_SCRATCH_BYTES,
+                            static_cast<hipStream_t>(stream));
+}
+
+int64_t sbnet_reduce_mask_static_max_indices(void)
+{
+    // the largest T with reduce_mask_workspace_bytes(T) <= STATIC_SCRATCH_BYTES
+    int64_t lo = 0, hi = (int64_t)sbnet::STATIC_SCRATCH_BYTES;
+    while (lo < hi) {
+        const int64_t mid = (lo + hi + 1) / 2;
+        if (sbnet::reduce_mask_workspace_bytes(mid) <= sbnet::STATIC_SCRATCH_BYTES) lo = mid;
+        else hi = mid - 1;
+    }
+    return lo;
 }
 
 int sbnet_reduce_mask_functor(const float* mask, int N, int H, int W, float threshold, int bOffsH0,

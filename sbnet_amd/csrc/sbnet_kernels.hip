@@ -21,6 +21,7 @@
 #include <stdint.h>
 
 #include <atomic>
+#include <mutex>
 
 #include "sbnet_launch.h"
 
@@ -1636,6 +1637,32 @@ int32_t* reduce_mask_count_slot(void* workspace, int64_t totalBlocks)
 {
     const size_t flags = ((size_t)totalBlocks + 15) & ~(size_t)15;
     return reinterpret_cast<int32_t*>(static_cast<uint8_t*>(workspace) + REDUCE_WORDS_BYTES + flags) + totalBlocks;
+}
+
+// Scratch for callers that can neither allocate nor bring a workspace (sbnet_reduce_mask_static): one array per
+// GPU, part of the loaded code object, held until the process ends.  Host code never passes the array's name to a
+// kernel: the name is a host-side stand-in, the device address comes from hipGetSymbolAddress, once per device.
+static __device__ __align__(256) __attribute__((used)) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
+hipError_t static_scratch(void** ptr)
+{
+    constexpr int MAX_DEVICES = 64;
+    static std::mutex mutex;
+    static void* ptrs[MAX_DEVICES] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= MAX_DEVICES) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(mutex);
+    if (!ptrs[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));  // of the current device's copy of the array
+        if (e != hipSuccess) return e;
+        if (!p) return hipErrorInvalidSymbol;
+        ptrs[dev] = p;
+    }
+    *ptr = ptrs[dev];
+    return hipSuccess;
 }
 
 static uint32_t next_reduce_tag()

@@ -37,6 +37,11 @@ hipError_t launch_reduce_mask(const float* mask, const Geom& g, int bCntH, int b
                               int32_t* binCountDevice, void* workspace, hipStream_t stream,
                               unsigned long long* hostSignal = nullptr, uint32_t hostSeq = 0);
 
+// Device address of the library's own scratch array on the current device (STATIC_SCRATCH_BYTES bytes, 256-byte
+// aligned): no allocation, looked up once per device.  Every call on a GPU shares that GPU's array.
+constexpr size_t STATIC_SCRATCH_BYTES = (size_t)2 << 20;
+hipError_t static_scratch(void** ptr);
+
 hipError_t launch_gather(const float* x, float* y, const int16_t* idx, int numActive,
                          const Geom& g, bool transpose, hipStream_t stream);
 
