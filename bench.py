@@ -15,10 +15,11 @@ The step is timed three ways (`pipeline` in the output): with the reference's ho
 (reduce_mask returns once the count has reached the host, which sizes the other launches), with the count left on the
 device (the `_device_count` entry points, three calls per step), and with those three launches captured
 in a HIP graph and replayed.  One JSON line goes to stdout.  `value` is algorithmic bytes per step /
-wall time per step with the count on the device (eager launches); the other two are reported beside
-it.  `ops`
-holds per-op device times (HIP events around batches of back-to-back launches on the launch stream),
-`roofline` the dominant kernel (the transposing gather) against the 8 TB/s HBM peak, `cpu_baseline`
+wall time per step under the reference's contract (host-visible count); the other two are reported beside
+it.  Each is the median of 15 batches of `--steps` steps.  `ops`
+holds per-op device times (HIP events around batches of back-to-back launches on the launch stream) at
+`--density`, `ops_by_density` the same at 5 %, 15 % and 30 %,
+`roofline` the dominant kernel (the slower of gather and scatter) against the 8 TB/s HBM peak, `cpu_baseline`
 the single-threaded CPU oracle (the reference's CPU functors restated; the reference builds them
 without OpenMP) on the same workload on this machine's host cores.  Tables for the other
 configurations (`--all-configs`) go to stderr.
@@ -242,6 +243,18 @@ class Path:
         if self.wl.x is not None:
             ops["gather"] = self.time_op(lambda i: self.gather(i, self.M))
         ops["scatter"] = self.time_op(lambda i: self.scatter(i, self.M))
+        wl = self.wl
+        if wl.s_var and not wl.s_add and (wl.s_bstride[0] < wl.s_bsize[0] or wl.s_bstride[1] < wl.s_bsize[1]):
+            # the same scatter given scratch: overlapping plain writes in the CPU functor's order (owner map built
+            # by two small launches, then the scatter with one owner read per pixel)
+            nsw = self.lib.sbnet_sparse_scatter_workspace_bytes(self.M, self.dims, 4, self.sbs, 2, self.sbst, 2,
+                                                                self.sbo, 2)
+            for s in self.sets:
+                s["sws"] = self.torch.empty(nsw, dtype=self.torch.uint8, device="cuda:0")
+            ops["scatter_ordered"] = self.time_op(lambda i: self.scatter(i, self.M))
+            self.bytes["scatter_ordered"] = self.bytes["scatter"]
+            for s in self.sets:
+                s["sws"] = None
         table = {}
         for k, us in ops.items():
             gbs = self.bytes[k] / us * 1e-3
@@ -299,19 +312,19 @@ def cpu_baseline(wl, M, idx_host, nbytes, budget_s=12.0):
              "ms_per_pass": round(tm * 1e3, 2)})
 
 
-def read_measured_traffic(name):
-    """HBM bytes per launch measured with rocprofv3 --pmc, if a summary under profiles/ records them as
-    lines `fetch_bytes_per_launch=<int>` and `write_bytes_per_launch=<int>`."""
+def read_measured_traffic(name, op):
+    """HBM bytes per launch of `op` ("gather" or "scatter") measured with rocprofv3 --pmc, if a summary under
+    profiles/ records them as lines `<op>_fetch_bytes_per_launch=<int>` and `<op>_write_bytes_per_launch=<int>`."""
     p = os.path.join(ROOT, "profiles", name)
     if not os.path.exists(p):
         return None
     vals = {}
     for line in open(p):
-        for key in ("fetch_bytes_per_launch", "write_bytes_per_launch"):
+        for key in ("%s_fetch_bytes_per_launch" % op, "%s_write_bytes_per_launch" % op):
             if line.strip().startswith(key + "="):
                 vals[key] = int(float(line.split("=", 1)[1].split()[0]))
     if len(vals) == 2:
-        return vals["fetch_bytes_per_launch"] + vals["write_bytes_per_launch"]
+        return sum(vals.values())
     return None
 
 
@@ -348,21 +361,39 @@ def main():
         print(json.dumps(config_row(args.only, torch, lib, workloads)))
         return
 
-    wl = workloads.config3(args.density)
-    path = Path(wl, torch, lib, nsets=3)
+    # per-op device times at the three densities the configuration sweeps; the buffers of the density the
+    # pipeline is timed on (--density) are kept for the step timings below
+    densities = sorted(set([0.05, 0.15, 0.30, args.density]))
+    ops_by_density = {}
+    path = None
+    for d in densities:
+        p = Path(workloads.config3(d), torch, lib, nsets=3)
+        table = p.op_table()
+        table["M"] = p.M
+        ops_by_density["%d%%" % round(d * 100)] = table
+        if d == args.density:
+            path, wl, ops = p, p.wl, table
+        else:
+            del p
+            torch.cuda.empty_cache()
     nsets = len(path.sets)
-    step_bytes = sum(path.bytes.values())
+    step_bytes = path.bytes["reduce_mask"] + path.bytes["gather"] + path.bytes["scatter"]
+    BATCHES = 15
 
     def timed(step_fn):
-        """W untimed steps, then exactly K steps between two device synchronisations; ms per step."""
+        """W untimed steps, then BATCHES batches of exactly K steps, each between two device synchronisations;
+        ms per step of the median batch (K steps of 0.1 ms are too short a sample to quote one batch)."""
         for i in range(max(args.warmup, nsets)):
             step_fn(i % nsets)
         torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for i in range(args.steps):
-            step_fn(i % nsets)
-        torch.cuda.synchronize()
-        return (time.perf_counter() - t0) / args.steps * 1e3
+        per = []
+        for b in range(BATCHES):
+            t0 = time.perf_counter()
+            for i in range(args.steps):
+                step_fn((b * args.steps + i) % nsets)
+            torch.cuda.synchronize()
+            per.append((time.perf_counter() - t0) / args.steps * 1e3)
+        return statistics.median(per)
 
     def variant(ms, note):
         return {"ms_per_step": round(ms, 4), "GBps": round(step_bytes / (ms * 1e-3) * 1e-9, 1), "note": note}
@@ -405,40 +436,51 @@ def main():
         s.pop("stack_cap", None)
     torch.cuda.empty_cache()
 
-    # `value`: the pipeline as this library is meant to be driven (count on the device, nothing waits for the
-    # host).  The reference's host-count contract and the graph replay are reported beside it.
-    ms_per_step = dc_ms
+    # `value`: the pipeline under the reference's contract (reduce_mask returns with the count on the host, gather
+    # and scatter are sized from it).  The variants that leave the count on the device are reported beside it.
+    ms_per_step = host_ms
     value = step_bytes / (ms_per_step * 1e-3) * 1e-9
 
-    ops = path.op_table()
-    g = ops["gather"]
-    roofline = {"bound": "hbm", "kernel": "k_gather_lines<5> (sparse_gather, transpose=True)",
+    # the dominant kernel: whichever of the two block movers takes longer per launch, in the launch shape `value`
+    # uses (grids sized from the host count, which is what the per-op table times)
+    dom = "gather" if ops["gather"]["us"] >= ops["scatter"]["us"] else "scatter"
+    g = ops[dom]
+    kernel_names = {"gather": "planar gather of sparse_gather(transpose=True): k_gather_lines",
+                    "scatter": "planar scatter of sparse_scatter_var(add=False, transpose=True): k_scatter_planar"}
+    traffic_file = "gather_lines_scatter_planar_C3_30pct_pmc.txt"
+    traffic = read_measured_traffic(traffic_file, dom) if round(args.density * 100) == 30 else None
+    roofline = {"bound": "hbm", "kernel": kernel_names[dom],
                 "achieved": g["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(g["GBps"] / HBM_PEAK_GBS, 4), "us_per_launch": g["us"],
                 "algorithmic_bytes_per_launch": g["bytes"],
-                "traffic": read_measured_traffic("gather_lines_scatter_planar_C3_30pct_pmc.txt")}
-    if roofline["traffic"]:
+                "traffic": traffic,
+                "traffic_source": ("profiles/%s (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by the copy kernel; "
+                                   "not re-measured by this run)" % traffic_file) if traffic else None}
+    if traffic:
         # the same launch time against the bytes the profiler counted between L2 and the fabric
-        roofline["traffic_GBps"] = round(roofline["traffic"] / g["us"] * 1e-3, 1)
+        roofline["traffic_GBps"] = round(traffic / g["us"] * 1e-3, 1)
     out = {
-        "metric": "achieved HBM GB/s over reduce_mask+sparse_gather+sparse_scatter_var (algorithmic bytes / wall time per step); us/op and % of HBM peak under ops and roofline",
+        "metric": "achieved HBM GB/s over reduce_mask+sparse_gather+sparse_scatter_var (algorithmic bytes / wall time per step); us/op and % of HBM peak under ops, ops_by_density and roofline",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "C3 LiDAR-BEV x=[1,800,800,128] fp32, bsize 27 bstride 25 boffset -1, max-pool tol 0.5, "
                                "%d%% of 1024 blocks active (M=%d), gather transpose=True, scatter_var add=False in place"
                                % (round(args.density * 100), path.M),
-                   "buffer_sets": nsets, "bytes_per_step": step_bytes},
-        "ops": ops, "roofline": roofline,
+                   "buffer_sets": nsets, "bytes_per_step": step_bytes,
+                   "timing": "median of %d batches of %d steps, each batch between two device synchronisations"
+                             % (BATCHES, args.steps)},
+        "ops": ops, "ops_by_density": ops_by_density, "roofline": roofline,
         "pipeline": {
-            "device_count_graph": variant(graph_ms, "count read on the device, reduce_mask + gather + scatter_var "
-                                                    "captured in one HIP graph per buffer set, one replay per step"),
-            "device_count_eager": variant(dc_ms, "value: count read on the device, three C-ABI calls per step from Python, "
-                                                 "launches sized for max_active=%d blocks" % path.maxidx),
-            "host_count_reference_contract": variant(host_ms, "reduce_mask returns with the count on the host "
+            "host_count_reference_contract": variant(host_ms, "value: reduce_mask returns with the count on the host "
                                                               "(the reference's HostMemory output; stored into "
                                                               "pinned memory by the kernel and polled), gather "
                                                               "and scatter sized from it"),
+            "device_count_eager": variant(dc_ms, "count read on the device (entry points only this library has), three "
+                                                 "C-ABI calls per step from Python, launches sized for max_active=%d "
+                                                 "blocks" % path.maxidx),
+            "device_count_graph": variant(graph_ms, "count read on the device, reduce_mask + gather + scatter_var "
+                                                    "captured in one HIP graph per buffer set, one replay per step"),
         },
     }
     if not args.no_cpu:

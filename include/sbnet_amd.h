@@ -126,8 +126,8 @@ int sbnet_reduce_mask(const float* mask, int N, int H, int W,
  *   beyond that the call returns SBNET_ETOOBIG and launches nothing.
  *   Every call on a GPU uses that GPU's one array: calls that may run at the same time on one GPU (different
  *   streams, different threads) race on it and must be serialised by the caller; calls on one stream are.
- *   Nothing in the array has to be cleared between calls (the kernel tells a call's data from what an earlier
- *   call left by a per-call tag), so a smaller problem may follow a larger one.
+ *   Nothing in the array has to be cleared between calls (every byte of it that a call reads has been
+ *   written by that call), so a smaller problem may follow a larger one.
  */
 int sbnet_reduce_mask_static(const float* mask, int N, int H, int W,
                              const int32_t* bcount, int bcount_len,

@@ -20,7 +20,6 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-#include <atomic>
 #include <mutex>
 
 #include "sbnet_launch.h"
@@ -1041,28 +1040,25 @@ __global__ __launch_bounds__(256) void k_planar_small(const float* __restrict__ 
 // reduce_mask: pooling + ordered stream compaction
 // ---------------------------------------------------------------------------------------------
 //
-// Pooling (k_reduce_pool): G = 2^logG lanes cooperate on one sparsity block (G grows with the
-// window, from 1 lane for tiny windows to a full wave) and decide "active".  Blocks are numbered
-// b = (n*bCntH + bh)*bCntW + bw, the order in which the CPU functor visits them
-// (reduce_mask.cc:71-73); a workgroup owns CH consecutive blocks.
+// Kernel 1 (k_reduce_pool): G = 2^logG lanes cooperate on one sparsity block (G grows with the
+// window, from 1 lane for tiny windows to a full wave), decide "active" and store one flag byte
+// per block plus one count per workgroup.  Blocks are numbered b = (n*bCntH + bh)*bCntW + bw,
+// the order in which the CPU functor visits them (reduce_mask.cc:71-73).
 //
-// Up to ONE_LAUNCH_MAX_BLOCKS blocks the whole op is this one launch.  Each workgroup publishes the
-// active bits of its blocks as 64-bit words (call tag << 32 | bits) with one atomic store each, then
-// reads all words of the grid; a workgroup that finds every word carrying the tag of this call knows
-// that the whole grid is done and holds every bit: it does the ordered compaction (popcount prefix
-// over the words, triples written in block order), the count, the "no active block" fix-up
-// (reduce_mask.cc:206-218) and the host-visible count, and finally zeroes the words.  Whichever
-// workgroup stores its words last always qualifies; two that finish together may both qualify and
-// then write the same values to the same places.  The tag makes the scheme independent of what the
-// scratch held before (nothing has to be cleared ahead of the launch, which a second launch would
-// cost); zeroing the words afterwards keeps a captured launch, which replays the same tag,
-// repeatable.  No workgroup ever waits for another.
+// Kernel 2 (k_reduce_compact): one thread per block; wave64 ballot + popcount gives the rank of
+// each active block inside its wave, LDS the wave offsets, the per-workgroup counts of kernel 1
+// the offset of the workgroup (summed by each workgroup while there are few; beyond
+// SCAN_MIN_COUNTS counts k_reduce_scan, one workgroup, turns them into exclusive prefix sums
+// first).  Triples therefore land in the CPU functor's order, and the last workgroup knows the
+// total: it stores the count and applies the "no active block" fix-up (reduce_mask.cc:206-218)
+// on the device.  Nothing in the scratch has to be cleared before a call: every byte that is
+// read has been written by the same call.
 //
-// Beyond that size: k_reduce_pool stores one flag byte per block and one count per workgroup,
-// k_reduce_scan (one workgroup, only for more than SCAN_MIN_COUNTS counts) turns the counts into
-// exclusive prefix sums, and k_reduce_compact (one thread per block; wave64 ballot + popcount for the
-// rank inside the wave, LDS for the wave offsets) writes the triples in order; its last workgroup
-// stores the count and applies the fix-up.
+// (A single launch, in which every workgroup publishes its bits in tagged words and the last one
+// to publish compacts, was measured and dropped: workgroups of one launch can only meet through
+// device-scope memory operations, and on this chip one such load takes about 2 us: 7.9 us per
+// launch against 6.7 us for the two launches; device-scope fences instead of atomic accesses
+// cost 30 us.)
 //
 // avg mode: the CPU functor adds the in-range pixels in row-major order (reduce_mask.cc:78-88)
 // and fp32 addition is not associative.  A cooperative sum is used only where it provably yields
@@ -1081,16 +1077,8 @@ struct PoolArgs {
     int logG;         // log2 of the lanes that share one block
     int passes;       // blocks per group
     FastDiv dBw, dBhw;
-    // one-launch mode (words != nullptr)
-    unsigned long long* words;  // nWords tagged words in the scratch
-    uint32_t tag;               // never 0
-    uint32_t nWords;
-    int wbLog;                  // log2 of the blocks per word: min(CH, 32)
-    int fixupZero;
 };
 
-constexpr uint32_t ONE_LAUNCH_MAX_BLOCKS = 16384;
-constexpr uint32_t ONE_LAUNCH_MAX_WORDS = 1024;   // 4 words per thread of a 256-thread workgroup
 constexpr uint32_t SCAN_MIN_COUNTS = 1024;
 
 // Stores the count (and, for an empty list, the (0,0,0) triple of reduce_mask.cc:206-218) and hands it to a
@@ -1124,16 +1112,11 @@ __device__ __forceinline__ float next_up(float f) { return -next_down(-f); }
 constexpr int POOL_LD = 8;  // loads in flight per lane
 
 __global__ __launch_bounds__(256) void k_reduce_pool(const float* __restrict__ mask, PoolArgs a,
-                                                     uint8_t* __restrict__ flags, int32_t* __restrict__ counts,
-                                                     int16_t* __restrict__ idx, int32_t* __restrict__ binCount,
-                                                     unsigned long long* hostSignal, uint32_t hostSeq)
+                                                     uint8_t* __restrict__ flags, int32_t* __restrict__ counts)
 {
     __shared__ int wgCount;
-    __shared__ uint32_t wgBits[8];  // one bit per block of this workgroup (at most 256)
-    __shared__ int scanWave[4];
     const uint32_t tid = threadIdx.x;
     if (tid == 0) wgCount = 0;
-    if (tid < 8) wgBits[tid] = 0u;
     __syncthreads();
 
     const int G = 1 << a.logG;
@@ -1230,96 +1213,12 @@ __global__ __launch_bounds__(256) void k_reduce_pool(const float* __restrict__ m
                     act = (s / denom) > a.tol;
                 }
             }
-            if (a.words) {
-                const uint32_t lb = (uint32_t)pass * groups + grp;  // position inside the workgroup's blocks
-                if (act) atomicOr(&wgBits[lb >> 5], 1u << (lb & 31u));
-            } else {
-                flags[b] = act ? 1 : 0;
-                if (act) atomicAdd(&wgCount, 1);
-            }
+            flags[b] = act ? 1 : 0;
+            if (act) atomicAdd(&wgCount, 1);
         }
     }
     __syncthreads();
-    if (!a.words) {
-        if (tid == 0) counts[blockIdx.x] = wgCount;
-        return;
-    }
-
-    // ---- one-launch mode: publish this workgroup's bits, then see whether the whole grid has published ----
-    {
-        const uint32_t WB = 1u << a.wbLog;
-        const uint32_t wordsPerWg = CH >> a.wbLog;  // CH / min(CH, 32)
-        if (tid < wordsPerWg) {
-            const uint32_t w = blockIdx.x * wordsPerWg + tid;
-            if (w < a.nWords) {
-                const uint32_t bits = WB == 32u ? wgBits[tid] : (wgBits[0] & ((1u << WB) - 1u));
-                __hip_atomic_store(a.words + w, ((unsigned long long)a.tag << 32) | bits, __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
-            }
-        }
-        // the stores above must be visible before this workgroup's loads below are performed: with that order
-        // on every workgroup, whichever stores last sees all the others
-        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "agent");
-        __syncthreads();
-        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "agent");
-
-        // thread t holds words [t*K, t*K + K): consecutive, so the prefix over threads is the prefix over blocks
-        constexpr uint32_t KMAX = ONE_LAUNCH_MAX_WORDS / 256;
-        const uint32_t K = (a.nWords + 255u) / 256u;
-        uint32_t bitsOf[KMAX];
-        int mine = 0;
-        bool tagged = true;
-#pragma unroll
-        for (uint32_t k = 0; k < KMAX; ++k) {
-            bitsOf[k] = 0u;
-            const uint32_t w = tid * K + k;
-            if (k < K && w < a.nWords) {
-                const unsigned long long v = __hip_atomic_load(a.words + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                tagged = tagged && (uint32_t)(v >> 32) == a.tag;
-                bitsOf[k] = (uint32_t)v;
-                mine += __popc(bitsOf[k]);
-            }
-        }
-        if (!__syncthreads_and(tagged ? 1 : 0)) return;  // some workgroup has not published yet: it will see us
-
-        // exclusive prefix of `mine` over the workgroup
-        const uint32_t lane = tid & 63u, wave = tid >> 6;
-        int incl = mine;
-        for (int off = 1; off < 64; off <<= 1) {
-            const int up = __shfl_up(incl, off);
-            if ((int)lane >= off) incl += up;
-        }
-        if (lane == 63u) scanWave[wave] = incl;
-        __syncthreads();
-        int pos = incl - mine;
-        for (uint32_t w = 0; w < wave; ++w) pos += scanWave[w];
-        const int total = scanWave[0] + scanWave[1] + scanWave[2] + scanWave[3];
-#pragma unroll
-        for (uint32_t k = 0; k < KMAX; ++k) {
-            uint32_t bits = bitsOf[k];
-            const uint32_t b0 = (tid * K + k) << a.wbLog;
-            while (bits) {
-                const uint32_t b = b0 + (uint32_t)__builtin_ctz(bits);
-                bits &= bits - 1u;
-                const uint32_t n = fdiv(b, a.dBhw);
-                const uint32_t rem = b - n * (uint32_t)(a.bCntH * a.bCntW);
-                const uint32_t bh = fdiv(rem, a.dBw);
-                int16_t* t = idx + (size_t)pos * 3;
-                t[0] = (int16_t)n;
-                t[1] = (int16_t)bh;
-                t[2] = (int16_t)(rem - bh * (uint32_t)a.bCntW);
-                ++pos;
-            }
-        }
-        if (tid == 0) publish_count(total, a.fixupZero, idx, binCount, hostSignal, hostSeq);
-        // leave the words without a tag: a replay of this launch from a captured graph carries the same tag
-#pragma unroll
-        for (uint32_t k = 0; k < KMAX; ++k) {
-            const uint32_t w = tid * K + k;
-            if (k < K && w < a.nWords)
-                __hip_atomic_store(a.words + w, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-    }
+    if (tid == 0) counts[blockIdx.x] = wgCount;
 }
 
 // Exclusive prefix sums of the pooling workgroups' counts, in place, by one workgroup of 1024 threads: each
@@ -1623,20 +1522,18 @@ static int pick_vec(const Geom& g, const void* a, const void* b)
     return 1;
 }
 
-// Scratch layout: the tagged words of the one-launch mode, then (larger problems) one flag byte per block, one
-// int32 count per pooling workgroup and the total for callers that give no device count.
-constexpr size_t REDUCE_WORDS_BYTES = (size_t)ONE_LAUNCH_MAX_WORDS * sizeof(unsigned long long);
-
+// Scratch layout: one flag byte per block (padded to 16), one int32 count per pooling workgroup (one per block
+// at worst), and the total for callers that give no device count.
 size_t reduce_mask_workspace_bytes(int64_t totalBlocks)
 {
     const size_t flags = ((size_t)totalBlocks + 15) & ~(size_t)15;
-    return REDUCE_WORDS_BYTES + flags + (size_t)totalBlocks * sizeof(int32_t) + 16;
+    return flags + (size_t)totalBlocks * sizeof(int32_t) + 16;
 }
 
 int32_t* reduce_mask_count_slot(void* workspace, int64_t totalBlocks)
 {
     const size_t flags = ((size_t)totalBlocks + 15) & ~(size_t)15;
-    return reinterpret_cast<int32_t*>(static_cast<uint8_t*>(workspace) + REDUCE_WORDS_BYTES + flags) + totalBlocks;
+    return reinterpret_cast<int32_t*>(static_cast<uint8_t*>(workspace) + flags) + totalBlocks;
 }
 
 // Scratch for callers that can neither allocate nor bring a workspace (sbnet_reduce_mask_static): one array per
@@ -1665,22 +1562,13 @@ hipError_t static_scratch(void** ptr)
     return hipSuccess;
 }
 
-static uint32_t next_reduce_tag()
-{
-    static std::atomic<uint32_t> counter{0};
-    uint32_t t = ++counter;
-    if (t == 0) t = ++counter;  // 0 marks a word that carries no call's bits
-    return t;
-}
-
 hipError_t launch_reduce_mask(const float* mask, const Geom& g, int bCntH, int bCntW, float tol,
                               bool avgPool, bool fixupZero, int16_t* activeBlockIndices,
                               int32_t* binCountDevice, void* workspace, hipStream_t stream,
                               unsigned long long* hostSignal, uint32_t hostSeq)
 {
     const uint32_t T = (uint32_t)((int64_t)g.N * bCntH * bCntW);
-    unsigned long long* words = static_cast<unsigned long long*>(workspace);
-    uint8_t* flags = static_cast<uint8_t*>(workspace) + REDUCE_WORDS_BYTES;
+    uint8_t* flags = static_cast<uint8_t*>(workspace);
     const size_t flagBytes = ((size_t)T + 15) & ~(size_t)15;
     int32_t* counts = reinterpret_cast<int32_t*>(flags + flagBytes);
     if (!binCountDevice) binCountDevice = reduce_mask_count_slot(workspace, T);
@@ -1710,21 +1598,7 @@ hipError_t launch_reduce_mask(const float* mask, const Geom& g, int bCntH, int b
     // the compaction relates pooling workgroups to its own 256 blocks, which needs CH to divide 256
     if (CH > 256) return hipErrorInvalidConfiguration;
 
-    p.wbLog = ilog2_floor(CH < 32u ? CH : 32u);
-    p.nWords = (T + (1u << p.wbLog) - 1u) >> p.wbLog;
-    p.fixupZero = fixupZero ? 1 : 0;
-    p.tag = 0;
-    p.words = nullptr;
-    if (T <= ONE_LAUNCH_MAX_BLOCKS && p.nWords <= ONE_LAUNCH_MAX_WORDS) {
-        p.words = words;
-        p.tag = next_reduce_tag();
-        hipLaunchKernelGGL(k_reduce_pool, dim3(nPool), dim3(256), 0, stream, mask, p, flags, counts, activeBlockIndices,
-                           binCountDevice, hostSignal, hostSeq);
-        return hipGetLastError();
-    }
-
-    hipLaunchKernelGGL(k_reduce_pool, dim3(nPool), dim3(256), 0, stream, mask, p, flags, counts, activeBlockIndices,
-                       binCountDevice, hostSignal, hostSeq);
+    hipLaunchKernelGGL(k_reduce_pool, dim3(nPool), dim3(256), 0, stream, mask, p, flags, counts);
     CompactArgs c;
     c.T = T;
     c.nCounts = nPool;

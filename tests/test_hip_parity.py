@@ -370,6 +370,29 @@ def test_reduce_mask_many_blocks_and_async_count():
     np.testing.assert_array_equal(host(r2.active_block_indices)[:int(cnt_o[0])], idx_o[:int(cnt_o[0])])
 
 
+def test_reduce_mask_four_million_blocks():
+    """N = 64 images of 256x256 one-pixel blocks: 4 194 304 blocks, 16 384 pooling workgroups whose counts go
+    through the prefix-sum kernel.  Order and count against the oracle, and the three launches take far less than
+    the time a compaction that re-sums all earlier counts in every workgroup would."""
+    rng = np.random.default_rng(77)
+    N, H, W = 64, 256, 256
+    mask = (rng.random((N, H, W, 1)) < 0.3).astype(np.float32)
+    bc, bs, bst, bo = [H, W], [1, 1], [1, 1], [0, 0]
+    idx_o, cnt_o = orc.reduce_mask(mask, bc, bs, bst, bo, 0.5, False)
+    M = int(cnt_o[0])
+    md = dev(mask)
+    r = sbnet_amd.reduce_mask(md, bc, bs, bst, bo, tol=0.5, avgpool=False)
+    assert int(r.bin_counts[0]) == M
+    assert torch.equal(r.active_block_indices[:M].cpu(), torch.from_numpy(idx_o[:M]))
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(5):
+        sbnet_amd.reduce_mask(md, bc, bs, bst, bo, tol=0.5, avgpool=False, sync=False)
+    e1.record()
+    e1.synchronize()
+    assert e0.elapsed_time(e1) / 5 < 5.0, "reduce_mask over 4M blocks took %.2f ms" % (e0.elapsed_time(e1) / 5)
+
+
 @pytest.mark.parametrize("bs,bst,bo", [((2, 2), (2, 2), (0, 0)), ((3, 3), (2, 2), (-1, -1))])
 def test_more_blocks_than_a_launch_dimension_holds(bs, bst, bo):
     """More than 65 535 active blocks: the planar kernels then number their workgroups along one launch
