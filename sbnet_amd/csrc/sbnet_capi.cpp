@@ -19,6 +19,7 @@
 namespace {
 
 thread_local int g_lastHipError = 0;
+thread_local int t_forceGeneric = 0;  // test hook, see sbnet_test_force_generic
 
 int hip_fail(hipError_t e)
 {
@@ -150,6 +151,7 @@ sbnet::Geom make_geom(int N, int H, int W, int C, const int32_t* bsize, const in
     g.U = bstride[0]; g.V = bstride[1];
     g.oh = boffset[0]; g.ow = boffset[1];
     g.countDev = nullptr;
+    g.forceGeneric = t_forceGeneric;
     return g;
 }
 
@@ -639,6 +641,16 @@ int sbnet_shutdown(void)
     }
     if (first != hipSuccess) return hip_fail(first);
     return SBNET_OK;
+}
+
+// Test hook, not part of the public header: while on (per calling thread), gather and scatter never take a
+// kernel instance compiled for one block shape, so the tests cover the run-time-geometry kernels on the
+// benchmark shapes as well.  Returns the previous setting.
+int sbnet_test_force_generic(int on)
+{
+    const int prev = t_forceGeneric;
+    t_forceGeneric = on ? 1 : 0;
+    return prev;
 }
 
 int sbnet_copy_tensor(float* dst, const float* src, size_t count, void* stream)

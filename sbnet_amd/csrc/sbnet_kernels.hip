@@ -373,7 +373,8 @@ struct TileArgs {
     int cchunks;        // channel chunks per block
     uint32_t tpb;       // tiles per block = psplit * cchunks
     uint32_t total;     // numActive * tpb
-    int grid2d;         // the launch is (tpb, numActive): the block is blockIdx.y and needs no division
+    int grid2d;         // the launch is (tpb, block rows): see for_each_block_of_workgroup
+    uint32_t blocks;    // capacity of the block list (numActive)
     uint32_t vpr;       // slots per planar row: (P + 3) / 4
     int64_t imgFloats;  // H * W * C
     uint32_t imgBytes;  // H * W * C * 4, below 2^32 (the host falls back to k_planar_small otherwise)
@@ -385,24 +386,65 @@ struct TileId {
     int c0, ctEff, p0, Pn;
 };
 
-// With a (tiles per block, blocks) launch the block number comes straight from the workgroup id, so the load
-// of its index triple can be issued from preloaded kernel arguments before anything else arrives.
-__device__ __forceinline__ void decode_tile(const TileArgs& a, TileId& t)
+// Geometry of a tile launch: read from the argument struct, or fixed at compile time (see LinesRt / LinesFixed
+// further down for what that buys).
+struct TileRt {
+    static constexpr bool FIXED = false;
+    __device__ static uint32_t nthr(const TileArgs&) { return blockDim.x; }
+    __device__ static uint32_t S(const TileArgs& a) { return (uint32_t)a.g.S; }
+    __device__ static uint32_t C(const TileArgs& a) { return (uint32_t)a.g.C; }
+    __device__ static uint32_t RS(const TileArgs& a) { return (uint32_t)(a.g.R * a.g.S); }
+    __device__ static uint32_t P(const TileArgs& a) { return (uint32_t)a.P; }
+    __device__ static uint32_t Pp(const TileArgs& a) { return (uint32_t)a.Pp; }
+    __device__ static uint32_t psplit(const TileArgs& a) { return (uint32_t)a.psplit; }
+    __device__ static uint32_t Ct(const TileArgs& a) { return (uint32_t)a.Ct; }
+    __device__ static uint32_t lppLog(const TileArgs& a) { return (uint32_t)a.lppLog; }
+    __device__ static uint32_t tpb(const TileArgs& a) { return a.tpb; }
+    __device__ static uint32_t vpr(const TileArgs& a) { return a.vpr; }
+    __device__ static uint32_t divS(uint32_t v, const TileArgs& a) { return fdiv(v, a.dS); }
+    __device__ static uint32_t divPs(uint32_t v, const TileArgs& a) { return fdiv(v, a.dPs); }
+    __device__ static uint32_t divTpb(uint32_t v, const TileArgs& a) { return fdiv(v, a.dTpb); }
+    __device__ static uint32_t divVpr(uint32_t v, const TileArgs& a) { return fdiv(v, a.dVpr); }
+};
+
+// 4-float channel vectors only (C_ a multiple of 4); P_ pixels per tile.
+template <int R_, int S_, int C_, int P_, int NTHR_>
+struct TileFixed {
+    static constexpr bool FIXED = true;
+    static constexpr uint32_t kRS = R_ * S_;
+    static constexpr uint32_t kLpp = C_ >= 32 ? 8 : C_ / 4;
+    static constexpr uint32_t kLppLog = kLpp == 8 ? 3 : kLpp == 4 ? 2 : kLpp == 2 ? 1 : 0;
+    static constexpr uint32_t kPsplit = (kRS + P_ - 1) / P_;
+    static constexpr uint32_t kPp = (P_ + 31) / 32 * 32;
+    static constexpr uint32_t kVpr = (P_ + 3) / 4;
+    static constexpr uint32_t kCchunks = (C_ + 4 * kLpp - 1) / (4 * kLpp);
+    __host__ __device__ static constexpr uint32_t nthr(const TileArgs&) { return NTHR_; }
+    __host__ __device__ static constexpr uint32_t S(const TileArgs&) { return S_; }
+    __host__ __device__ static constexpr uint32_t C(const TileArgs&) { return C_; }
+    __host__ __device__ static constexpr uint32_t RS(const TileArgs&) { return kRS; }
+    __host__ __device__ static constexpr uint32_t P(const TileArgs&) { return P_; }
+    __host__ __device__ static constexpr uint32_t Pp(const TileArgs&) { return kPp; }
+    __host__ __device__ static constexpr uint32_t psplit(const TileArgs&) { return kPsplit; }
+    __host__ __device__ static constexpr uint32_t Ct(const TileArgs&) { return 4 * kLpp; }
+    __host__ __device__ static constexpr uint32_t lppLog(const TileArgs&) { return kLppLog; }
+    __host__ __device__ static constexpr uint32_t tpb(const TileArgs&) { return kPsplit * kCchunks; }
+    __host__ __device__ static constexpr uint32_t vpr(const TileArgs&) { return kVpr; }
+    __host__ __device__ static constexpr uint32_t divS(uint32_t v, const TileArgs&) { return v / (uint32_t)S_; }
+    __host__ __device__ static constexpr uint32_t divPs(uint32_t v, const TileArgs&) { return v / kPsplit; }
+    __host__ __device__ static constexpr uint32_t divTpb(uint32_t v, const TileArgs&) { return v / (kPsplit * kCchunks); }
+    __host__ __device__ static constexpr uint32_t divVpr(uint32_t v, const TileArgs&) { return v / kVpr; }
+};
+
+template <typename G>
+__device__ __forceinline__ void decode_tile(const TileArgs& a, TileId& t, uint32_t ib, uint32_t rem)
 {
-    uint32_t rem;
-    if (a.grid2d) {
-        t.ib = blockIdx.y;
-        rem = blockIdx.x;
-    } else {
-        t.ib = fdiv(blockIdx.x, a.dTpb);
-        rem = blockIdx.x - t.ib * a.tpb;
-    }
-    const uint32_t cc = fdiv(rem, a.dPs);
-    const uint32_t pc = rem - cc * (uint32_t)a.psplit;
-    t.c0 = (int)cc * a.Ct;
-    t.ctEff = min(a.Ct, a.g.C - t.c0);
-    t.p0 = (int)pc * a.P;
-    t.Pn = min(a.P, a.g.R * a.g.S - t.p0);
+    t.ib = ib;
+    const uint32_t cc = G::divPs(rem, a);
+    const uint32_t pc = rem - cc * G::psplit(a);
+    t.c0 = (int)(cc * G::Ct(a));
+    t.ctEff = (int)min(G::Ct(a), G::C(a) - (uint32_t)t.c0);
+    t.p0 = (int)(pc * G::P(a));
+    t.Pn = (int)min(G::P(a), G::RS(a) - (uint32_t)t.p0);
 }
 
 __device__ __forceinline__ uint32_t lds_swz(uint32_t c) { return ((c >> 2) & 7u) << 2; }
@@ -587,29 +629,30 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
 // u = 0 .. TILE_LD-1, pl0 = tid >> lppLog, step = nthr >> lppLog.  Walks those pixels keeping (r, s) by
 // increments and hands each one's byte offset inside the image (or BUF_OOB) and its pixel number h*W + w (only
 // meaningful with an in-range offset) to `f(u, pl, off, pix)`.
-template <int VEC, typename F>
+template <int VEC, typename G, typename F>
 __device__ __forceinline__ void nhwc_walk(const TileArgs& a, const TileId& t, const BlockOrigin& o, uint32_t tid,
                                           uint32_t nthr, F f)
 {
-    const uint32_t lppMask = (1u << a.lppLog) - 1u;
-    const uint32_t step = nthr >> a.lppLog;
-    const uint32_t stepR = fdiv(step, a.dS), stepS = step - stepR * (uint32_t)a.g.S;
-    uint32_t pl = tid >> a.lppLog;
-    const int c = t.c0 + (int)(tid & lppMask) * VEC;
+    const uint32_t lppLog = G::lppLog(a), S = G::S(a), C = G::C(a);
+    const uint32_t lppMask = (1u << lppLog) - 1u;
+    const uint32_t step = nthr >> lppLog;
+    const uint32_t stepR = G::divS(step, a), stepS = step - stepR * S;
+    uint32_t pl = tid >> lppLog;
+    const uint32_t c = (uint32_t)t.c0 + (tid & lppMask) * VEC;
     const uint32_t p = (uint32_t)t.p0 + pl;
-    uint32_t r = fdiv(p, a.dS), s = p - r * (uint32_t)a.g.S;
-    const bool cok = c < a.g.C;
+    uint32_t r = G::divS(p, a), s = p - r * S;
+    const bool cok = c < C;
 #pragma unroll
     for (int u = 0; u < TILE_LD; ++u) {
         const int hh = o.h0 + (int)r, ww = o.w0 + (int)s;
         const bool ok = cok && pl < (uint32_t)t.Pn && (unsigned)hh < (unsigned)a.g.H && (unsigned)ww < (unsigned)a.g.W;
-        const uint32_t off = (((uint32_t)hh * (uint32_t)a.g.W + (uint32_t)ww) * (uint32_t)a.g.C + (uint32_t)c) * 4u;
+        const uint32_t off = (((uint32_t)hh * (uint32_t)a.g.W + (uint32_t)ww) * C + c) * 4u;
         f(u, pl, ok ? off : BUF_OOB, (uint32_t)hh * (uint32_t)a.g.W + (uint32_t)ww);
         pl += step;
         r += stepR;
         s += stepS;
-        if (s >= (uint32_t)a.g.S) {
-            s -= (uint32_t)a.g.S;
+        if (s >= S) {
+            s -= S;
             ++r;
         }
     }
@@ -617,15 +660,15 @@ __device__ __forceinline__ void nhwc_walk(const TileArgs& a, const TileId& t, co
 
 // sparse_gather.cc:67-88 with transpose == true: y[ib, c, r, s] = x[n, h0+r, w0+s, c] or 0.
 template <int VEC>
-__global__ __launch_bounds__(512) void k_gather_planar(const float* __restrict__ x, float* __restrict__ y,
-                                                       const int16_t* __restrict__ idx, TileArgs a)
+__device__ __forceinline__ void gather_planar_tile(const float* __restrict__ x, float* __restrict__ y,
+                                                   const int16_t* __restrict__ idx, const TileArgs& a, float* lds,
+                                                   uint32_t ib, uint32_t rem)
 {
     typedef typename Vec<VEC>::type vec;
-    extern __shared__ __attribute__((aligned(16))) float lds[];
     const uint32_t tid = threadIdx.x, nthr = blockDim.x;
     const uint32_t RS = (uint32_t)(a.g.R * a.g.S);
     TileId t;
-    decode_tile(a, t);
+    decode_tile<TileRt>(a, t, ib, rem);
     const RawTriple raw = load_triple(idx, t.ib);
     if (beyond_count(a.g, t.ib)) return;
     const BlockOrigin o = origin_of(raw, a.g);
@@ -634,7 +677,7 @@ __global__ __launch_bounds__(512) void k_gather_planar(const float* __restrict__
 
     vec v[TILE_LD];
     uint32_t pls[TILE_LD];
-    nhwc_walk<VEC>(a, t, o, tid, nthr, [&](int u, uint32_t pl, uint32_t off, uint32_t) {
+    nhwc_walk<VEC, TileRt>(a, t, o, tid, nthr, [&](int u, uint32_t pl, uint32_t off, uint32_t) {
         v[u] = buf_load<VEC>(xr, off);
         pls[u] = pl;
     });
@@ -684,6 +727,16 @@ __global__ __launch_bounds__(512) void k_gather_planar(const float* __restrict__
     }
 }
 
+template <int VEC>
+__global__ __launch_bounds__(512) void k_gather_planar(const float* __restrict__ x, float* __restrict__ y,
+                                                       const int16_t* __restrict__ idx, TileArgs a)
+{
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    for_each_block_of_workgroup(a, a.tpb, [&](uint32_t ib, uint32_t rem) {
+        gather_planar_tile<VEC>(x, y, idx, a, lds, ib, rem);
+    });
+}
+
 // ---------------------------------------------------------------------------------------------
 // Planar gather whose workgroups own whole 128-byte lines of the output
 // ---------------------------------------------------------------------------------------------
@@ -718,8 +771,8 @@ struct LineArgs {
     int Ct, lppLog;
     int RS;
     int P, Pp, psplit, cchunks;
-    int ext;            // window pixels beyond the tile's own: LINE_EXT
-    int grid2d;         // the launch is (tpb, numActive): the block is blockIdx.y
+    int grid2d;         // the launch is (tpb, block rows): see for_each_block_of_workgroup
+    uint32_t blocks;    // capacity of the block list (numActive)
     uint32_t tpb, total;
     uint32_t spr;       // bound on the output slots of one row of one tile
     int64_t imgFloats;
@@ -727,48 +780,92 @@ struct LineArgs {
     FastDiv dTpb, dPs, dS;
 };
 
-template <int LD>
-__global__ __launch_bounds__(512) void k_gather_lines(const float* __restrict__ x, float* __restrict__ y,
-                                                      const int16_t* __restrict__ idx, LineArgs a)
-{
-    extern __shared__ __attribute__((aligned(16))) float lds[];
-    const uint32_t tid = threadIdx.x, nthr = blockDim.x;
-    const uint32_t RS = (uint32_t)a.RS;
+// Geometry of a launch as the kernels see it: either read from the argument struct (any shape) or fixed at compile
+// time for the shapes the benchmark configurations use.  With constants the reciprocal divisions, the pitch
+// multiplications and the pixel-step bookkeeping fold away (about a third of the vector instructions of a tile),
+// LDS accesses take immediate offsets and the unused staging variants are not compiled in.  The host launches a
+// fixed-shape instance only when the tile it chose equals the instance's (sbnet_launch.h: Geom::forceGeneric keeps
+// tests on the run-time path).
+struct LinesRt {
+    static constexpr bool FIXED = false;
+    __device__ static uint32_t nthr(const LineArgs&) { return blockDim.x; }
+    __device__ static uint32_t R(const LineArgs& a) { return (uint32_t)a.g.R; }
+    __device__ static uint32_t S(const LineArgs& a) { return (uint32_t)a.g.S; }
+    __device__ static uint32_t C(const LineArgs& a) { return (uint32_t)a.g.C; }
+    __device__ static uint32_t RS(const LineArgs& a) { return (uint32_t)a.RS; }
+    __device__ static uint32_t P(const LineArgs& a) { return (uint32_t)a.P; }
+    __device__ static uint32_t Pp(const LineArgs& a) { return (uint32_t)a.Pp; }
+    __device__ static uint32_t psplit(const LineArgs& a) { return (uint32_t)a.psplit; }
+    __device__ static uint32_t Ct(const LineArgs& a) { return (uint32_t)a.Ct; }
+    __device__ static uint32_t lppLog(const LineArgs& a) { return (uint32_t)a.lppLog; }
+    __device__ static uint32_t tpb(const LineArgs& a) { return a.tpb; }
+    __device__ static uint32_t divS(uint32_t v, const LineArgs& a) { return fdiv(v, a.dS); }
+    __device__ static uint32_t divPs(uint32_t v, const LineArgs& a) { return fdiv(v, a.dPs); }
+    __device__ static uint32_t divTpb(uint32_t v, const LineArgs& a) { return fdiv(v, a.dTpb); }
+};
 
-    uint32_t ib, rem;
-    if (a.grid2d) {
-        ib = blockIdx.y;
-        rem = blockIdx.x;
-    } else {
-        ib = fdiv(blockIdx.x, a.dTpb);
-        rem = blockIdx.x - ib * a.tpb;
-    }
+template <int R_, int S_, int C_, int PSPLIT_, int NTHR_>
+struct LinesFixed {
+    static constexpr bool FIXED = true;
+    static constexpr uint32_t kRS = R_ * S_;
+    static constexpr uint32_t kLpp = C_ >= 32 ? 8 : C_ / 4;  // C_ a multiple of 4; Ct = min(C_, 32) rounded to 2^k*4
+    static constexpr uint32_t kLppLog = kLpp == 8 ? 3 : kLpp == 4 ? 2 : kLpp == 2 ? 1 : 0;
+    static constexpr uint32_t kP = (kRS + PSPLIT_ - 1) / PSPLIT_;
+    static constexpr uint32_t kPp = (kP + LINE_EXT + 3 + 31) / 32 * 32;
+    static constexpr uint32_t kCchunks = (C_ + 4 * kLpp - 1) / (4 * kLpp);
+    static constexpr int kLD = (int)(((kP + LINE_EXT) * kLpp + NTHR_ - 1) / NTHR_) < 4
+                                   ? 4 : (int)(((kP + LINE_EXT) * kLpp + NTHR_ - 1) / NTHR_);
+    __host__ __device__ static constexpr uint32_t nthr(const LineArgs&) { return NTHR_; }
+    __host__ __device__ static constexpr uint32_t R(const LineArgs&) { return R_; }
+    __host__ __device__ static constexpr uint32_t S(const LineArgs&) { return S_; }
+    __host__ __device__ static constexpr uint32_t C(const LineArgs&) { return C_; }
+    __host__ __device__ static constexpr uint32_t RS(const LineArgs&) { return kRS; }
+    __host__ __device__ static constexpr uint32_t P(const LineArgs&) { return kP; }
+    __host__ __device__ static constexpr uint32_t Pp(const LineArgs&) { return kPp; }
+    __host__ __device__ static constexpr uint32_t psplit(const LineArgs&) { return PSPLIT_; }
+    __host__ __device__ static constexpr uint32_t Ct(const LineArgs&) { return 4 * kLpp; }
+    __host__ __device__ static constexpr uint32_t lppLog(const LineArgs&) { return kLppLog; }
+    __host__ __device__ static constexpr uint32_t tpb(const LineArgs&) { return PSPLIT_ * kCchunks; }
+    __host__ __device__ static constexpr uint32_t divS(uint32_t v, const LineArgs&) { return v / (uint32_t)S_; }
+    __host__ __device__ static constexpr uint32_t divPs(uint32_t v, const LineArgs&) { return v / (uint32_t)PSPLIT_; }
+    __host__ __device__ static constexpr uint32_t divTpb(uint32_t v, const LineArgs&) { return v / (PSPLIT_ * kCchunks); }
+};
+
+template <int LD, typename G>
+__device__ __forceinline__ void gather_lines_tile(const float* __restrict__ x, float* __restrict__ y,
+                                                  const int16_t* __restrict__ idx, const LineArgs& a, float* lds,
+                                                  uint32_t ib, uint32_t rem)
+{
+    const uint32_t tid = threadIdx.x, nthr = G::nthr(a);
+    const uint32_t RS = G::RS(a), S = G::S(a), R = G::R(a), C = G::C(a), Pp = G::Pp(a);
+    const uint32_t lppLog = G::lppLog(a);
+
     const RawTriple raw = load_triple(idx, ib);
     if (beyond_count(a.g, ib)) return;
-    const uint32_t cc = fdiv(rem, a.dPs);
-    const uint32_t split = rem - cc * (uint32_t)a.psplit;
-    const uint32_t c0 = cc * (uint32_t)a.Ct;
-    const uint32_t ctEff = min((uint32_t)a.Ct, (uint32_t)a.g.C - c0);
-    const uint32_t p0 = split * (uint32_t)a.P;
-    const uint32_t p1 = min(p0 + (uint32_t)a.P, RS);
-    const uint32_t win = p1 - p0 + (uint32_t)a.ext;
+    const uint32_t cc = G::divPs(rem, a);
+    const uint32_t split = rem - cc * G::psplit(a);
+    const uint32_t c0 = cc * G::Ct(a);
+    const uint32_t ctEff = min(G::Ct(a), C - c0);
+    const uint32_t p0 = split * G::P(a);
+    const uint32_t p1 = min(p0 + G::P(a), RS);
+    const uint32_t win = p1 - p0 + (uint32_t)LINE_EXT;
 
     const BlockOrigin o = origin_of(raw, a.g);
     const rsrc_t xr = make_rsrc(x + (o.valid ? (int64_t)o.n * a.imgFloats : 0), o.valid ? a.imgBytes : 0u);
 
     // NHWC side: lane owns channels [4*cl, 4*cl + 4) of window pixels q0 + u*step.  (r, s) of the pixel is
     // kept by increments; stepping past the end of the plane wraps to its start, which is r -= R.
-    const uint32_t cl = tid & ((1u << a.lppLog) - 1u);
-    const uint32_t q0 = tid >> a.lppLog, step = nthr >> a.lppLog;
+    const uint32_t cl = tid & ((1u << lppLog) - 1u);
+    const uint32_t q0 = tid >> lppLog, step = nthr >> lppLog;
     const uint32_t c = c0 + cl * 4u;
-    const bool cok = c < (uint32_t)a.g.C;
-    const uint32_t stepR = fdiv(step, a.dS), stepS = step - stepR * (uint32_t)a.g.S;
+    const bool cok = c < C;
+    const uint32_t stepR = G::divS(step, a), stepS = step - stepR * S;
     uint32_t r, sc;
     {
         uint32_t p = p0 + q0;
         if (p >= RS) p -= RS;
-        r = fdiv(p, a.dS);
-        sc = p - r * (uint32_t)a.g.S;
+        r = G::divS(p, a);
+        sc = p - r * S;
     }
     f4 v[LD];
 #pragma unroll
@@ -776,15 +873,15 @@ __global__ __launch_bounds__(512) void k_gather_lines(const float* __restrict__ 
         const uint32_t q = q0 + (uint32_t)u * step;
         const int hh = o.h0 + (int)r, ww = o.w0 + (int)sc;
         const bool ok = cok && q < win && (unsigned)hh < (unsigned)a.g.H && (unsigned)ww < (unsigned)a.g.W;
-        const uint32_t off = (((uint32_t)hh * (uint32_t)a.g.W + (uint32_t)ww) * (uint32_t)a.g.C + c) * 4u;
+        const uint32_t off = (((uint32_t)hh * (uint32_t)a.g.W + (uint32_t)ww) * C + c) * 4u;
         v[u] = buf_load<4>(xr, ok ? off : BUF_OOB);
         sc += stepS;
         r += stepR;
-        if (sc >= (uint32_t)a.g.S) {
-            sc -= (uint32_t)a.g.S;
+        if (sc >= S) {
+            sc -= S;
             ++r;
         }
-        if (r >= (uint32_t)a.g.R) r -= (uint32_t)a.g.R;
+        if (r >= R) r -= R;
     }
     // registers -> LDS.  In the last split of a plane the window wraps: its pixels from `wrapStart` on are the
     // first pixels of the plane, which the output needs as the continuation of the PREVIOUS channel's row (the
@@ -799,7 +896,7 @@ __global__ __launch_bounds__(512) void k_gather_lines(const float* __restrict__ 
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             const uint32_t phi = ((uint32_t)k * RS + p0) & 3u;  // == ((4*cl + k)*RS + p0) & 3
-            rowAddr[k] = (cl * 4u + (uint32_t)k) * (uint32_t)a.Pp + phi;
+            rowAddr[k] = (cl * 4u + (uint32_t)k) * Pp + phi;
         }
         if ((step & 31u) == 0) {
 #pragma unroll
@@ -830,10 +927,10 @@ __global__ __launch_bounds__(512) void k_gather_lines(const float* __restrict__ 
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             const uint32_t phi = ((uint32_t)k * RS + p0) & 3u;
-            rowAddr[k] = (cl * 4u + (uint32_t)k) * (uint32_t)a.Pp + ((phi + q0) ^ swz);
+            rowAddr[k] = (cl * 4u + (uint32_t)k) * Pp + ((phi + q0) ^ swz);
         }
         const uint32_t rowP = cl * 4u - 1u;  // no such row for cl == 0: channel 0 drops its wrapped pixels
-        const uint32_t addrP = rowP * (uint32_t)a.Pp + ((((rowP * RS + p0) & 3u) + q0) ^ lds_swz(rowP));
+        const uint32_t addrP = rowP * Pp + ((((rowP * RS + p0) & 3u) + q0) ^ lds_swz(rowP));
 #pragma unroll
         for (int u = 0; u < LD; ++u) {
             const uint32_t q = q0 + (uint32_t)u * step;
@@ -854,7 +951,7 @@ __global__ __launch_bounds__(512) void k_gather_lines(const float* __restrict__ 
                 for (int k = 0; k < 4; ++k) {
                     const uint32_t row = cl * 4u + (uint32_t)k - back;  // 0xFFFFFFFF for channel 0's wrapped pixels
                     const uint32_t phi = (row * RS + p0) & 3u;
-                    if (row != 0xFFFFFFFFu) lds[row * (uint32_t)a.Pp + ((phi + q) ^ lds_swz(row))] = vget(v[u], k);
+                    if (row != 0xFFFFFFFFu) lds[row * Pp + ((phi + q) ^ lds_swz(row))] = vget(v[u], k);
                 }
             }
         }
@@ -862,7 +959,7 @@ __global__ __launch_bounds__(512) void k_gather_lines(const float* __restrict__ 
     lds_barrier();
 
     // planar side: whole lines of the chunk
-    const int64_t chunkBase = ((int64_t)ib * a.g.C + c0) * RS;
+    const int64_t chunkBase = ((int64_t)ib * C + c0) * RS;
     const uint32_t chunkFloats = ctEff * RS;
     const uint32_t a0 = (uint32_t)(((reinterpret_cast<uintptr_t>(y) >> 2) + (uint64_t)chunkBase) & (LINE_FLOATS - 1));
     const rsrc_t yr = make_rsrc(y + chunkBase, chunkFloats * 4u);
@@ -888,7 +985,7 @@ __global__ __launch_bounds__(512) void k_gather_lines(const float* __restrict__ 
                     const uint32_t l = A + k4;
                     const bool live = l < B;
                     // (a row's last line may run into the next plane: those pixels sit behind the row in LDS)
-                    qv[u] = lds_read4(lds + (live ? cr * (uint32_t)a.Pp + ((colBase + k4) ^ lds_swz(cr)) : 0u));
+                    qv[u] = lds_read4(lds + (live ? cr * Pp + ((colBase + k4) ^ lds_swz(cr)) : 0u));
                     off[u] = live ? l * 4u : BUF_OOB;
                 }
 #pragma unroll
@@ -898,17 +995,52 @@ __global__ __launch_bounds__(512) void k_gather_lines(const float* __restrict__ 
     }
 }
 
+// Launch shapes of the tile kernels.  (tiles per block, block rows): the block is the workgroup's y id, so its
+// index triple can be fetched from preloaded kernel arguments before anything else arrives.  With the block count
+// in device memory the launch cannot be sized for it: it covers half of the list's capacity in block rows and a
+// workgroup takes block y and, if that is below the count, block y + rows.  Lists are rarely more than half full
+// (sparse blocks pay off below that), so a workgroup almost never takes a second block, and the workgroups
+// of rows past the count, which leave after one scalar load, are halved (at capacity 1024 and 312 blocks 17 088
+// of them cost the scatter 3.6 us).  Beyond 65 535 block rows the launch is linear over the tiles.
+template <typename ARGS, typename F>
+__device__ __forceinline__ void for_each_block_of_workgroup(const ARGS& a, uint32_t tpb, F tile)
+{
+    if (a.grid2d) {
+        // (two calls, not a loop: around a loop the compiler kept the whole tile's address arithmetic live and
+        // tripled the register count)
+        tile(blockIdx.y, blockIdx.x);
+        const uint32_t ib2 = blockIdx.y + gridDim.y;
+        if (ib2 < a.blocks && !beyond_count(a.g, ib2)) {  // (the same for the whole workgroup)
+            __syncthreads();                               // LDS is reused
+            tile(ib2, blockIdx.x);
+        }
+    } else {
+        const uint32_t ib = blockIdx.x / tpb;
+        tile(ib, blockIdx.x - ib * tpb);
+    }
+}
+
+template <int LD, typename G>
+__global__ __launch_bounds__(512) void k_gather_lines(const float* __restrict__ x, float* __restrict__ y,
+                                                      const int16_t* __restrict__ idx, LineArgs a)
+{
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    for_each_block_of_workgroup(a, G::tpb(a), [&](uint32_t ib, uint32_t rem) {
+        gather_lines_tile<LD, G>(x, y, idx, a, lds, ib, rem);
+    });
+}
+
 // sparse_gather.cc:103-130 with transpose == true: the block stack is [blocks, C, R, S].
-template <int VEC, int MODE>
-__global__ __launch_bounds__(512) void k_scatter_planar(const float* __restrict__ x, float* y, const float* ysrc,
-                                                        const int16_t* __restrict__ idx, TileArgs a, ColorArgs col)
+template <int VEC, int MODE, typename G>
+__device__ __forceinline__ void scatter_planar_tile(const float* __restrict__ x, float* y, const float* ysrc,
+                                                    const int16_t* __restrict__ idx, const TileArgs& a,
+                                                    const ColorArgs& col, float* lds, uint32_t ib, uint32_t rem)
 {
     typedef typename Vec<VEC>::type vec;
-    extern __shared__ __attribute__((aligned(16))) float lds[];
-    const uint32_t tid = threadIdx.x, nthr = blockDim.x;
-    const uint32_t RS = (uint32_t)(a.g.R * a.g.S);
+    const uint32_t tid = threadIdx.x, nthr = G::nthr(a);
+    const uint32_t RS = G::RS(a), Pp = G::Pp(a), vpr = G::vpr(a);
     TileId t;
-    decode_tile(a, t);
+    decode_tile<G>(a, t, ib, rem);
     const RawTriple raw = load_triple(idx, t.ib);  // scalar load, needed only after the barrier
     if (beyond_count(a.g, t.ib)) return;
     bool atomics = MODE == SCATTER_ATOMIC;
@@ -916,25 +1048,25 @@ __global__ __launch_bounds__(512) void k_scatter_planar(const float* __restrict_
 
     // global -> registers, planar side.  The last slot of a run, when partial, is read as the last 4 floats
     // of the run instead (overlapping its neighbour): no load leaves the run, no value needs fixing up.
-    const rsrc_t xr = make_rsrc(x + ((int64_t)t.ib * a.g.C + t.c0) * RS + t.p0,
+    const rsrc_t xr = make_rsrc(x + ((int64_t)t.ib * G::C(a) + t.c0) * RS + t.p0,
                                 ((uint32_t)(t.ctEff - 1) * RS + (uint32_t)t.Pn) * 4u);
-    const uint32_t slots = (uint32_t)t.ctEff * a.vpr;
+    const uint32_t slots = (uint32_t)t.ctEff * vpr;
     if (t.Pn >= 4) {
         f4 val[TILE_LD];
 #pragma unroll
         for (int u = 0; u < TILE_LD; ++u) {
             const uint32_t i = u * nthr + tid;
-            const uint32_t c = fdiv(i, a.dVpr);
-            const int e0 = min(4 * (int)(i - c * a.vpr), t.Pn - 4);
+            const uint32_t c = G::divVpr(i, a);
+            const int e0 = min(4 * (int)(i - c * vpr), t.Pn - 4);
             val[u] = buf_load<4>(xr, i < slots ? (c * RS + (uint32_t)e0) * 4u : BUF_OOB);
         }
 #pragma unroll
         for (int u = 0; u < TILE_LD; ++u) {
             const uint32_t i = u * nthr + tid;
             if (i < slots) {
-                const uint32_t c = fdiv(i, a.dVpr);
-                const int e0 = 4 * (int)(i - c * a.vpr);
-                float* __restrict__ row = lds + c * a.Pp;
+                const uint32_t c = G::divVpr(i, a);
+                const int e0 = 4 * (int)(i - c * vpr);
+                float* __restrict__ row = lds + c * Pp;
                 if (e0 + 4 <= t.Pn) {
                     *reinterpret_cast<f4*>(row + ((uint32_t)e0 ^ lds_swz(c))) = val[u];
                 } else if (e0 < t.Pn) {  // partial last slot: holds floats [Pn-4, Pn) of the run
@@ -951,7 +1083,7 @@ __global__ __launch_bounds__(512) void k_scatter_planar(const float* __restrict_
         // and 1-3 pixels may remain): one thread per row moves them float by float.
         if (tid < (uint32_t)t.ctEff) {
             for (int k = 0; k < t.Pn; ++k)
-                lds[tid * a.Pp + ((uint32_t)k ^ lds_swz(tid))] = buf_load<1>(xr, (tid * RS + (uint32_t)k) * 4u);
+                lds[tid * Pp + ((uint32_t)k ^ lds_swz(tid))] = buf_load<1>(xr, (tid * RS + (uint32_t)k) * 4u);
         }
     }
     lds_barrier();
@@ -962,13 +1094,13 @@ __global__ __launch_bounds__(512) void k_scatter_planar(const float* __restrict_
     float* img = y + (int64_t)o.n * a.imgFloats;
     const rsrc_t yr = make_rsrc(img, a.imgBytes);
     const rsrc_t sr = make_rsrc(ysrc + (int64_t)o.n * a.imgFloats, a.imgBytes);  // what an add reads
-    const uint32_t c0l = (tid & ((1u << a.lppLog) - 1u)) * VEC;
+    const uint32_t c0l = (tid & ((1u << G::lppLog(a)) - 1u)) * VEC;
     vec w[TILE_LD];
     uint32_t offs[TILE_LD];
     int32_t own[TILE_LD];
     const rsrc_t wr = make_rsrc(MODE == SCATTER_OWNED ? col.owner + (int64_t)o.n * a.g.H * a.g.W : nullptr,
                                 MODE == SCATTER_OWNED ? (uint32_t)(a.g.H * a.g.W) * 4u : 0u);
-    nhwc_walk<VEC>(a, t, o, tid, nthr, [&](int u, uint32_t pl, uint32_t off, uint32_t pix) {
+    nhwc_walk<VEC, G>(a, t, o, tid, nthr, [&](int u, uint32_t pl, uint32_t off, uint32_t pix) {
         offs[u] = off;
         if (MODE == SCATTER_OWNED) own[u] = __builtin_bit_cast(int32_t, buf_load<1>(wr, off != BUF_OOB ? pix * 4u : BUF_OOB));
         w[u] = vzero<VEC>();
@@ -976,7 +1108,7 @@ __global__ __launch_bounds__(512) void k_scatter_planar(const float* __restrict_
 #pragma unroll
             for (int k = 0; k < VEC; ++k) {
                 const uint32_t c = c0l + k;
-                vset(w[u], k, lds[c * a.Pp + (pl ^ lds_swz(c))]);
+                vset(w[u], k, lds[c * Pp + (pl ^ lds_swz(c))]);
             }
         }
     });
@@ -1002,6 +1134,16 @@ __global__ __launch_bounds__(512) void k_scatter_planar(const float* __restrict_
             }
         }
     }
+}
+
+template <int VEC, int MODE, typename G>
+__global__ __launch_bounds__(512) void k_scatter_planar(const float* __restrict__ x, float* y, const float* ysrc,
+                                                        const int16_t* __restrict__ idx, TileArgs a, ColorArgs col)
+{
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    for_each_block_of_workgroup(a, G::tpb(a), [&](uint32_t ib, uint32_t rem) {
+        scatter_planar_tile<VEC, MODE, G>(x, y, ysrc, idx, a, col, lds, ib, rem);
+    });
 }
 
 // Fallback for block planes of fewer than 4 pixels (1x1, 1x2, 1x3 ... blocks), where a dwordx4 slot does
@@ -1508,10 +1650,12 @@ static int ilog2_floor(uint32_t v)
 
 constexpr int GRID_Y_MAX = 65535;
 
-// One workgroup per tile, as (tiles per block, blocks) when the block count fits the y dimension of a launch.
-static dim3 tile_grid(int grid2d, uint32_t tpb, int numActive, uint32_t total)
+// One workgroup per tile, as (tiles per block, block rows) when the block count fits the y dimension of a launch;
+// half as many rows as the list holds when the count is only known on the device (for_each_block_of_workgroup).
+static dim3 tile_grid(int grid2d, uint32_t tpb, int numActive, uint32_t total, const Geom& g)
 {
-    return grid2d ? dim3(tpb, (unsigned)numActive) : dim3(total);
+    if (!grid2d) return dim3(total);
+    return dim3(tpb, (unsigned)(g.countDev && numActive > 1 ? (numActive + 1) / 2 : numActive));
 }
 
 static int pick_vec(const Geom& g, const void* a, const void* b)
@@ -1690,13 +1834,61 @@ static bool make_tile_args(const Geom& g, int numActive, int vec, TileArgs& a, i
     if (ldsBytes > 64 * 1024) return false;
     grid = a.total;
     a.grid2d = numActive <= GRID_Y_MAX;
+    a.blocks = (uint32_t)numActive;
+    return true;
+}
+
+// Compute units of the current device (256 on MI355X), looked up once per device.
+static int device_cus()
+{
+    static std::mutex mutex;
+    static int cus[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+        (void)hipGetLastError();
+        return 256;
+    }
+    std::lock_guard<std::mutex> lock(mutex);
+    if (!cus[dev]) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+            (void)hipGetLastError();
+            n = 256;
+        }
+        cus[dev] = n;
+    }
+    return cus[dev];
+}
+
+// Tile of the planar scatter.  16 KB tiles suit a launch that keeps every compute unit busy for several
+// rounds of workgroups; a launch of few workgroups finishes in one or two rounds, where the loads and the stores
+// of one round do not overlap much, and does better with 24 KB tiles (800x800x128 tensor, 27x27 blocks:
+// 9.08 -> 8.87 us at 58 blocks, 20.6 -> 19.9 us at 156, but 40.8 -> 41.4 us at 312).
+constexpr int SCATTER_FEW_WGS_PER_CU = 22;
+
+static bool scatter_tile_args(const Geom& g, int numActive, int vec, TileArgs& a, int& threads, size_t& ldsBytes,
+                              unsigned& grid)
+{
+    if (!make_tile_args(g, numActive, vec, a, threads, ldsBytes, grid, 16 * 1024)) return false;
+    if (a.psplit > 1 && a.total < (uint32_t)(SCATTER_FEW_WGS_PER_CU * device_cus())) {
+        TileArgs b;
+        int bt;
+        size_t bl;
+        unsigned bg;
+        if (make_tile_args(g, numActive, vec, b, bt, bl, bg, 24 * 1024) && b.psplit < a.psplit) {
+            a = b;
+            threads = bt;
+            ldsBytes = bl;
+            grid = bg;
+        }
+    }
     return true;
 }
 
 // Tile choice of k_gather_lines.  Returns false where the kernel does not apply (the caller then uses
 // k_gather_planar): y not 16-byte aligned, a last split shorter than the window extension, LDS.
 static bool make_line_args(const Geom& g, int numActive, const float* y, LineArgs& a, int& threads, int& ld,
-                           size_t& ldsBytes, unsigned& grid)
+                           size_t& ldsBytes, unsigned& grid, int maxLd)
 {
     if (g.C % 4 != 0 || (reinterpret_cast<uintptr_t>(y) & 15) != 0) return false;
     a.g = g;
@@ -1712,8 +1904,7 @@ static bool make_line_args(const Geom& g, int numActive, const float* y, LineArg
     a.lppLog = ilog2_floor((uint32_t)lpp);
     a.cchunks = (g.C + a.Ct - 1) / a.Ct;
     // The smallest workgroup whose LD vectors per thread cover a whole plane; otherwise 512 threads and as
-    // few splits as the window (own pixels + LINE_EXT) allows within 5 vectors per thread.
-    const int maxLd = 5;
+    // few splits as the window (own pixels + LINE_EXT) allows within maxLd vectors per thread.
     threads = 0;
     a.psplit = 1;
     for (int nthr = 64; nthr <= 512; nthr *= 2) {
@@ -1729,9 +1920,8 @@ static bool make_line_args(const Geom& g, int numActive, const float* y, LineArg
     a.psplit = (RS + a.P - 1) / a.P;
     // A tile that takes whole planes writes one contiguous piece of y in k_gather_planar already.
     if (a.psplit == 1) return false;
-    a.ext = LINE_EXT;
     if (RS - (a.psplit - 1) * a.P < LINE_FLOATS) return false;  // the last split must hold the extension
-    const int win = a.P + a.ext;
+    const int win = a.P + LINE_EXT;
     ld = (win * lpp + threads - 1) / threads;
     if (ld < 4) ld = 4;
     if (ld > 8) return false;
@@ -1752,7 +1942,95 @@ static bool make_line_args(const Geom& g, int numActive, const float* y, LineArg
     a.dS = make_fastdiv((uint32_t)g.S);
     grid = a.total;
     a.grid2d = numActive <= GRID_Y_MAX;
+    a.blocks = (uint32_t)numActive;
     return true;
+}
+
+// 5 vectors per thread (three splits of a 27x27 plane) for launches of many workgroups, 7 (two splits: fewer
+// window pixels read twice, more bytes in flight per workgroup) for launches of few, as for the scatter:
+// 8.62 -> 7.76 us at 58 blocks, 21.7 -> 20.8 us at 156, but 40.3 -> 40.6 us at 312.
+constexpr int GATHER_FEW_WGS_PER_CU = 11;
+
+static bool choose_line_args(const Geom& g, int numActive, const float* y, LineArgs& a, int& threads, int& ld,
+                             size_t& ldsBytes, unsigned& grid)
+{
+    if (!make_line_args(g, numActive, y, a, threads, ld, ldsBytes, grid, 5)) return false;
+    if (a.total < (uint32_t)(GATHER_FEW_WGS_PER_CU * device_cus())) {
+        LineArgs b;
+        int bt, bld;
+        size_t bl;
+        unsigned bg;
+        if (make_line_args(g, numActive, y, b, bt, bld, bl, bg, 7) && b.psplit < a.psplit) {
+            a = b;
+            threads = bt;
+            ld = bld;
+            ldsBytes = bl;
+            grid = bg;
+        }
+    }
+    return true;
+}
+
+// Fixed-shape instances: launched when the run-time tile choice equals the instance's.
+template <typename G>
+static bool lines_match(const LineArgs& a, int threads, int ld)
+{
+    return !a.g.forceGeneric && a.g.R * a.g.S == (int)G::kRS && a.g.S == (int)G::S(a) && a.g.C == (int)G::C(a) &&
+           a.psplit == (int)G::psplit(a) && threads == (int)G::nthr(a) && a.P == (int)G::kP && a.Pp == (int)G::kPp &&
+           a.Ct == (int)G::Ct(a) && a.lppLog == (int)G::kLppLog && ld == G::kLD && a.tpb == G::tpb(a);
+}
+
+template <typename G>
+static bool launch_fixed_lines_one(const float* x, float* y, const int16_t* idx, const LineArgs& a, int threads, int ld,
+                                   size_t lds, int numActive, hipStream_t stream)
+{
+    if (!lines_match<G>(a, threads, ld)) return false;
+    hipLaunchKernelGGL((k_gather_lines<G::kLD, G>), tile_grid(a.grid2d, a.tpb, numActive, a.total, a.g), dim3(threads), lds,
+                       stream, x, y, idx, a);
+    return true;
+}
+
+static bool launch_fixed_lines(const float* x, float* y, const int16_t* idx, const LineArgs& a, int threads, int ld,
+                               size_t lds, int numActive, hipStream_t stream)
+{
+    // 27x27 blocks of 128 channels (800x800x128 tensor): three and two splits per plane; 18x18 blocks of 64 channels
+    return launch_fixed_lines_one<LinesFixed<27, 27, 128, 3, 512>>(x, y, idx, a, threads, ld, lds, numActive, stream) ||
+           launch_fixed_lines_one<LinesFixed<27, 27, 128, 2, 512>>(x, y, idx, a, threads, ld, lds, numActive, stream) ||
+           launch_fixed_lines_one<LinesFixed<18, 18, 64, 2, 512>>(x, y, idx, a, threads, ld, lds, numActive, stream);
+}
+
+template <typename G>
+static bool tile_match(const TileArgs& a, int threads)
+{
+    return !a.g.forceGeneric && a.g.R * a.g.S == (int)G::kRS && a.g.S == (int)G::S(a) && a.g.C == (int)G::C(a) &&
+           a.P == (int)G::P(a) && a.psplit == (int)G::kPsplit && threads == (int)G::nthr(a) && a.Pp == (int)G::kPp &&
+           a.Ct == (int)G::Ct(a) && a.lppLog == (int)G::kLppLog && a.vpr == G::kVpr && a.tpb == G::tpb(a);
+}
+
+template <int VEC, int MODE, typename G>
+static bool launch_fixed_scatter_one(const float* x, float* y, const float* ysrc, const int16_t* idx, const TileArgs& a,
+                                     int threads, size_t lds, int numActive, const ColorArgs& aux, hipStream_t stream)
+{
+    if (!tile_match<G>(a, threads)) return false;
+    hipLaunchKernelGGL((k_scatter_planar<VEC, MODE, G>), tile_grid(a.grid2d, a.tpb, numActive, a.total, a.g), dim3(threads),
+                       lds, stream, x, y, ysrc, idx, a, aux);
+    return true;
+}
+
+template <int VEC, int MODE>
+static bool launch_fixed_scatter(const float* x, float* y, const float* ysrc, const int16_t* idx, const TileArgs& a,
+                                 int threads, size_t lds, int numActive, const ColorArgs& aux, hipStream_t stream)
+{
+    if constexpr (VEC == 4 && (MODE == SCATTER_ASSIGN || MODE == SCATTER_ADD)) {
+        // 27x27 blocks of 128 channels with 16 KB and 24 KB tiles; 16x16 blocks of 64 channels
+        return launch_fixed_scatter_one<VEC, MODE, TileFixed<27, 27, 128, 124, 512>>(x, y, ysrc, idx, a, threads, lds,
+                                                                                      numActive, aux, stream) ||
+               launch_fixed_scatter_one<VEC, MODE, TileFixed<27, 27, 128, 184, 512>>(x, y, ysrc, idx, a, threads, lds,
+                                                                                      numActive, aux, stream) ||
+               launch_fixed_scatter_one<VEC, MODE, TileFixed<16, 16, 64, 128, 512>>(x, y, ysrc, idx, a, threads, lds,
+                                                                                     numActive, aux, stream);
+    }
+    return false;
 }
 
 template <int VEC>
@@ -1774,14 +2052,15 @@ static void gather_dispatch(const float* x, float* y, const int16_t* idx, const 
         if (VEC == 4) {
             LineArgs la;
             int ld;
-            if (make_line_args(g, numActive, y, la, threads, ld, lds, grid)) {
-                const dim3 lg = tile_grid(la.grid2d, la.tpb, numActive, la.total);
+            if (choose_line_args(g, numActive, y, la, threads, ld, lds, grid)) {
+                if (launch_fixed_lines(x, y, idx, la, threads, ld, lds, numActive, stream)) return;
+                const dim3 lg = tile_grid(la.grid2d, la.tpb, numActive, la.total, la.g);
                 switch (ld) {
-                case 4: hipLaunchKernelGGL(k_gather_lines<4>, lg, dim3(threads), lds, stream, x, y, idx, la); break;
-                case 5: hipLaunchKernelGGL(k_gather_lines<5>, lg, dim3(threads), lds, stream, x, y, idx, la); break;
-                case 6: hipLaunchKernelGGL(k_gather_lines<6>, lg, dim3(threads), lds, stream, x, y, idx, la); break;
-                case 7: hipLaunchKernelGGL(k_gather_lines<7>, lg, dim3(threads), lds, stream, x, y, idx, la); break;
-                default: hipLaunchKernelGGL(k_gather_lines<8>, lg, dim3(threads), lds, stream, x, y, idx, la); break;
+                case 4: hipLaunchKernelGGL((k_gather_lines<4, LinesRt>), lg, dim3(threads), lds, stream, x, y, idx, la); break;
+                case 5: hipLaunchKernelGGL((k_gather_lines<5, LinesRt>), lg, dim3(threads), lds, stream, x, y, idx, la); break;
+                case 6: hipLaunchKernelGGL((k_gather_lines<6, LinesRt>), lg, dim3(threads), lds, stream, x, y, idx, la); break;
+                case 7: hipLaunchKernelGGL((k_gather_lines<7, LinesRt>), lg, dim3(threads), lds, stream, x, y, idx, la); break;
+                default: hipLaunchKernelGGL((k_gather_lines<8, LinesRt>), lg, dim3(threads), lds, stream, x, y, idx, la); break;
                 }
                 return;
             }
@@ -1795,7 +2074,7 @@ static void gather_dispatch(const float* x, float* y, const int16_t* idx, const 
                                dim3(256), 0, stream, x, y, (const float*)y, idx, g, total, (const int32_t*)nullptr);
             return;
         }
-        hipLaunchKernelGGL(k_gather_planar<VEC>, tile_grid(a.grid2d, a.tpb, numActive, a.total), dim3(threads), lds,
+        hipLaunchKernelGGL(k_gather_planar<VEC>, tile_grid(a.grid2d, a.tpb, numActive, a.total, a.g), dim3(threads), lds,
                            stream, x, y, idx, a);
     }
 }
@@ -1837,15 +2116,16 @@ static void scatter_dispatch(const float* x, float* y, const float* ysrc, const 
         size_t lds;
         unsigned grid;
         // 16 KB tiles: 42.6 us against 43.9 us with 32 KB tiles on the same workload
-        if ((int64_t)g.R * g.S < 4 || !make_tile_args(g, numActive, VEC, a, threads, lds, grid, 16 * 1024)) {
+        if ((int64_t)g.R * g.S < 4 || !scatter_tile_args(g, numActive, VEC, a, threads, lds, grid)) {
             const int64_t total = (int64_t)numActive * g.C * g.R * g.S;
             const int64_t wgs = (total + 255) / 256;
             hipLaunchKernelGGL((k_planar_small<MODE, false>), dim3((unsigned)(wgs > 65536 ? 65536 : wgs)), dim3(256),
                                0, stream, x, y, ysrc, idx, g, total, owner);
             return;
         }
-        hipLaunchKernelGGL((k_scatter_planar<VEC, MODE>), tile_grid(a.grid2d, a.tpb, numActive, a.total), dim3(threads),
-                           lds, stream, x, y, ysrc, idx, a, aux);
+        if (launch_fixed_scatter<VEC, MODE>(x, y, ysrc, idx, a, threads, lds, numActive, aux, stream)) return;
+        hipLaunchKernelGGL((k_scatter_planar<VEC, MODE, TileRt>), tile_grid(a.grid2d, a.tpb, numActive, a.total, a.g),
+                           dim3(threads), lds, stream, x, y, ysrc, idx, a, aux);
     }
 }
 
@@ -1999,9 +2279,9 @@ static bool color_passes(const float* x, float* y, const int16_t* idx, const Geo
         int threads;
         size_t lds;
         unsigned grid;
-        if ((int64_t)g.R * g.S < 4 || !make_tile_args(g, numActive, VEC, a, threads, lds, grid, 16 * 1024)) return false;
+        if ((int64_t)g.R * g.S < 4 || !scatter_tile_args(g, numActive, VEC, a, threads, lds, grid)) return false;
         for (col.pass = 0; col.pass < passes; ++col.pass)
-            hipLaunchKernelGGL((k_scatter_planar<VEC, SCATTER_COLOR>), tile_grid(a.grid2d, a.tpb, numActive, a.total),
+            hipLaunchKernelGGL((k_scatter_planar<VEC, SCATTER_COLOR, TileRt>), tile_grid(a.grid2d, a.tpb, numActive, a.total, a.g),
                                dim3(threads), lds, stream, x, y, (const float*)y, idx, a, col);
     }
     return true;
@@ -2035,7 +2315,7 @@ hipError_t launch_scatter_colored(const float* x, float* y, const int16_t* idx, 
         size_t lds;
         unsigned grid;
         if (!transpose ? !make_nhwc_args(g, numActive, vec, na)
-                       : ((int64_t)g.R * g.S < 4 || !make_tile_args(g, numActive, vec, ta, threads, lds, grid, 16 * 1024)))
+                       : ((int64_t)g.R * g.S < 4 || !scatter_tile_args(g, numActive, vec, ta, threads, lds, grid)))
             return hipSuccess;
     }
     int64_t fillWgs = (mapN + 255) / 256;

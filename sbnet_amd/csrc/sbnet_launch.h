@@ -19,6 +19,9 @@ struct Geom {
     // capacity of the list and skip rows at or beyond *countDev, so no host round trip is needed between
     // reduce_mask and its consumers.
     const int32_t* countDev;
+    // Tests only: never launch a fixed-shape kernel instance, so that the run-time-geometry kernels are covered
+    // for the shapes that have instances too.
+    int forceGeneric;
 };
 
 enum ScatterMode { SCATTER_ASSIGN = 0, SCATTER_ADD = 1, SCATTER_ATOMIC = 2 };

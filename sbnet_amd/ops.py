@@ -199,8 +199,10 @@ def gather_forward(x, bin_counts, active_block_indices, dynamic_bsize, dynamic_b
 
 
 def scatter_forward(x, bin_counts, active_block_indices, ybase, dynamic_bsize, dynamic_bstride, dynamic_boffset, add,
-                    atomic, transpose, use_var):
-    """The scatter without autograd bookkeeping."""
+                    atomic, transpose, use_var, scratch=True):
+    """The scatter without autograd bookkeeping.  scratch=False passes no workspace to the library (hardware
+    atomics for overlapping adds, unordered overlapping plain writes, copy-then-scatter): what a caller of the
+    C ABI gets who brings none."""
     lib = _lib.load()
     x = _dev_f32(x, "x")
     idx = _idx_i16(active_block_indices)
@@ -221,7 +223,7 @@ def scatter_forward(x, bin_counts, active_block_indices, ybase, dynamic_bsize, d
         _check_stack(x, M, int(ybase.shape[3]), int(bs[0]), int(bs[1]), transpose, "x")
     with torch.cuda.device(ybase.device):
         ws_ptr, ws_bytes = None, 0
-        if (add and atomic) or not use_var or (not add and overlap):
+        if scratch and ((add and atomic) or not use_var or (not add and overlap)):
             # scratch for the atomic-free scatter-add of overlapping blocks, for overlapping plain writes in the
             # CPU functor's order (the block listed last wins), and for building the copying op's output in one
             # pass (uncovered pixels copied, covered ones scattered)
