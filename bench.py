@@ -11,12 +11,13 @@ than 1 GB in total) are rotated so the 256 MB Infinity Cache cannot serve one st
 All calls go through the C ABI of libsbnet_amd.so with ctypes; PyTorch only owns the device buffers
 and the stream.
 
-The step is timed three ways (`pipeline` in the output): with the reference's host-visible count
+The step is timed several ways (`pipeline` in the output): with the reference's host-visible count
 (reduce_mask returns once the count has reached the host, which sizes the other launches), with the count left on the
-device (the `_device_count` entry points, three calls per step), and with those three launches captured
+device (the `_device_count` entry points, three calls per step), each driven from a C++ host loop
+(libsbnet_bench.so, built from sbnet_amd/csrc/sbnet_bench_loop.cpp) and from Python, and with the three launches captured
 in a HIP graph and replayed.  One JSON line goes to stdout.  `value` is algorithmic bytes per step /
-wall time per step under the reference's contract (host-visible count); the other two are reported beside
-it.  Each is the median of 15 batches of `--steps` steps.  `ops`
+wall time per step under the reference's contract (host-visible count) from the C++ loop; the others are reported
+beside it.  Each is the median of 15 batches of `--steps` steps.  `ops`
 holds per-op device times (HIP events around batches of back-to-back launches on the launch stream) at
 `--density`, `ops_by_density` the same at 5 %, 15 % and 30 %,
 `roofline` the dominant kernel (the slower of gather and scatter) against the 8 TB/s HBM peak, `cpu_baseline`
@@ -57,6 +58,9 @@ def parse():
                     help="time one configuration only (C1, C2, C3@5%%, C3@15%%, C3@30%%, C4, C5) and print its row to "
                          "stdout instead of the benchmark line: for profiling the other configurations' kernels")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline (profiling runs)")
+    ap.add_argument("--ops-only", action="store_true",
+                    help="per-op tables only (ops_by_density), no pipeline timing: a kernel trace of this run holds "
+                         "exactly the launches the per-op times and the roofline come from")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run the library's plain copy kernel on 256 MiB, 10 times: a kernel of known traffic "
                          "against which profiler byte counters are scaled")
@@ -263,6 +267,58 @@ class Path:
         return table
 
 
+class BenchSet(ctypes.Structure):   # struct sbnet_bench_set of sbnet_amd/csrc/sbnet_bench_loop.cpp
+    _fields_ = [("mask", ctypes.c_void_p), ("x", ctypes.c_void_p), ("base", ctypes.c_void_p),
+                ("stack", ctypes.c_void_p), ("idx", ctypes.c_void_p), ("count_dev", ctypes.c_void_p),
+                ("reduce_ws", ctypes.c_void_p), ("reduce_ws_bytes", ctypes.c_size_t)]
+
+
+class BenchGeom(ctypes.Structure):  # struct sbnet_bench_geom
+    _fields_ = [("N", ctypes.c_int), ("H", ctypes.c_int), ("W", ctypes.c_int), ("C", ctypes.c_int),
+                ("bcount", I2), ("bsize", I2), ("bstride", I2), ("boffset", I2),
+                ("s_bsize", I2), ("s_bstride", I2), ("s_boffset", I2),
+                ("tol", ctypes.c_float), ("avgpool", ctypes.c_int), ("transpose", ctypes.c_int),
+                ("add", ctypes.c_int), ("atomic", ctypes.c_int), ("max_active", ctypes.c_int32)]
+
+
+def cxx_pipeline(path, steps, warmup, batches):
+    """The step driven by a C++ host loop over the same C ABI (libsbnet_bench.so): ms per step of the median batch,
+    for the reference's contract (mode 0, count handed to the host) and with the count on the device (mode 1)."""
+    so = os.path.join(ROOT, "sbnet_amd", "libsbnet_bench.so")
+    if not os.path.exists(so):
+        raise RuntimeError("%s is not built; run `make -C sbnet_amd/csrc`" % so)
+    loop = ctypes.CDLL(so).sbnet_bench_pipeline
+    loop.restype = ctypes.c_int
+    loop.argtypes = [ctypes.POINTER(BenchSet), ctypes.c_int, ctypes.POINTER(BenchGeom), ctypes.c_int, ctypes.c_int,
+                     ctypes.c_void_p, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int32)]
+    wl, torch = path.wl, path.torch
+    R, S = wl.bsize
+    caps = [torch.empty((path.maxidx, path.C, R, S) if wl.transpose else (path.maxidx, R, S, path.C),
+                        dtype=torch.float32, device="cuda:0") for _ in path.sets]
+    sets = (BenchSet * len(path.sets))()
+    for k, s in enumerate(path.sets):
+        sets[k] = BenchSet(s["mask"].data_ptr(), s["x"].data_ptr(), s["base"].data_ptr(), caps[k].data_ptr(),
+                           s["idx"].data_ptr(), s["dcount"].data_ptr(), s["ws"].data_ptr(), path.nws)
+    g = BenchGeom(path.N, path.H, path.W, path.C, I2(*wl.bcount), I2(*wl.bsize), I2(*wl.bstride), I2(*wl.boffset),
+                  I2(*wl.s_bsize), I2(*wl.s_bstride), I2(*wl.s_boffset), wl.tol, int(wl.avgpool), int(wl.transpose),
+                  int(wl.s_add), int(wl.s_atomic), path.maxidx)
+    out = {}
+    sec, cnt = ctypes.c_double(0.0), ctypes.c_int32(0)
+    for mode, name in ((0, "host_count"), (1, "device_count")):
+        path.check(loop(sets, len(path.sets), ctypes.byref(g), max(warmup, len(path.sets)), mode, path.stream,
+                        ctypes.byref(sec), ctypes.byref(cnt)))
+        per = []
+        for _ in range(batches):
+            path.check(loop(sets, len(path.sets), ctypes.byref(g), steps, mode, path.stream, ctypes.byref(sec),
+                            ctypes.byref(cnt)))
+            assert cnt.value == path.M, "active block count changed between runs"
+            per.append(sec.value / steps * 1e3)
+        out[name] = statistics.median(per)
+    del caps
+    torch.cuda.empty_cache()
+    return out
+
+
 def cpu_baseline(wl, M, idx_host, nbytes, budget_s=12.0):
     """Times the CPU oracle's gather + scatter (single thread: the reference's Makefile has no -fopenmp)
     on the same workload, repeating until about `budget_s` seconds have been spent."""
@@ -376,6 +432,9 @@ def main():
         else:
             del p
             torch.cuda.empty_cache()
+    if args.ops_only:
+        print(json.dumps({"ops_by_density": ops_by_density}))
+        return
     nsets = len(path.sets)
     step_bytes = path.bytes["reduce_mask"] + path.bytes["gather"] + path.bytes["scatter"]
     BATCHES = 15
@@ -436,9 +495,12 @@ def main():
         s.pop("stack_cap", None)
     torch.cuda.empty_cache()
 
+    # (4) the first two again from a C++ host loop: what a caller written in the reference's host language sees
+    cxx = cxx_pipeline(path, args.steps, args.warmup, BATCHES)
+
     # `value`: the pipeline under the reference's contract (reduce_mask returns with the count on the host, gather
-    # and scatter are sized from it).  The variants that leave the count on the device are reported beside it.
-    ms_per_step = host_ms
+    # and scatter are sized from it), driven from C++.  The other variants are reported beside it.
+    ms_per_step = cxx["host_count"]
     value = step_bytes / (ms_per_step * 1e-3) * 1e-9
 
     # the dominant kernel: whichever of the two block movers takes longer per launch, in the launch shape `value`
@@ -472,13 +534,18 @@ def main():
                              % (BATCHES, args.steps)},
         "ops": ops, "ops_by_density": ops_by_density, "roofline": roofline,
         "pipeline": {
-            "host_count_reference_contract": variant(host_ms, "value: reduce_mask returns with the count on the host "
-                                                              "(the reference's HostMemory output; stored into "
-                                                              "pinned memory by the kernel and polled), gather "
-                                                              "and scatter sized from it"),
-            "device_count_eager": variant(dc_ms, "count read on the device (entry points only this library has), three "
-                                                 "C-ABI calls per step from Python, launches sized for max_active=%d "
-                                                 "blocks" % path.maxidx),
+            "host_count_reference_contract_cxx": variant(cxx["host_count"],
+                                                         "value: reduce_mask returns with the count on the host (the "
+                                                         "reference's HostMemory output; stored into pinned memory by "
+                                                         "the kernel and polled), gather and scatter sized from it; "
+                                                         "three C-ABI calls per step from a C++ loop "
+                                                         "(sbnet_amd/csrc/sbnet_bench_loop.cpp)"),
+            "device_count_cxx": variant(cxx["device_count"], "count read on the device (entry points only this library "
+                                                             "has), launches sized for max_active=%d blocks, same "
+                                                             "C++ loop" % path.maxidx),
+            "host_count_reference_contract": variant(host_ms, "the reference's contract with the three calls made "
+                                                              "from Python through ctypes"),
+            "device_count_eager": variant(dc_ms, "count read on the device, three calls per step from Python"),
             "device_count_graph": variant(graph_ms, "count read on the device, reduce_mask + gather + scatter_var "
                                                     "captured in one HIP graph per buffer set, one replay per step"),
         },
