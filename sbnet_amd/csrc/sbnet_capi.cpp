@@ -653,6 +653,16 @@ int sbnet_test_force_generic(int on)
     return prev;
 }
 
+// Test hook, not part of the public header: the tile the planar kernels would choose (no device work, so the
+// choice can be checked on a machine without a GPU).  out must hold 11 int32; see sbnet::tile_choice.
+int sbnet_test_tile_choice(int kind, int N, int H, int W, int C, int R, int S, int U, int V, int num_active, int vec,
+                           int y_aligned_to, int32_t* out)
+{
+    const int32_t bsize[2] = {R, S}, bstride[2] = {U, V}, boffset[2] = {0, 0};
+    if (!out || !geom_ok(N, H, W, C, bsize, bstride)) return -1;
+    return sbnet::tile_choice(kind, make_geom(N, H, W, C, bsize, bstride, boffset), num_active, vec, y_aligned_to, out);
+}
+
 int sbnet_copy_tensor(float* dst, const float* src, size_t count, void* stream)
 {
     if (count && (!dst || !src)) return SBNET_EINVAL_ARG;

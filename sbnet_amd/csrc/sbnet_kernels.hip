@@ -2079,6 +2079,51 @@ static void gather_dispatch(const float* x, float* y, const int16_t* idx, const 
     }
 }
 
+// Test hook (sbnet_test_tile_choice): the tile the planar kernels would use for a geometry, without launching.
+// kind 0: k_gather_lines, 1: k_gather_planar, 2: k_scatter_planar.  out = {threads, ldsBytes, P, Pp, psplit, Ct,
+// cchunks, vectors or slots per thread needed, vectors or slots per thread available, last split's pixels, fixed
+// instance available}.  Returns 0 when that kernel does not apply to the geometry.
+int tile_choice(int kind, const Geom& g, int numActive, int vec, int yAlignedTo, int32_t* out)
+{
+    int threads = 0;
+    size_t lds = 0;
+    unsigned grid = 0;
+    const int RS = g.R * g.S;
+    if (kind == 0) {
+        LineArgs a;
+        int ld = 0;
+        // a y pointer with the requested alignment (never dereferenced)
+        const float* y = reinterpret_cast<const float*>((uintptr_t)0x10000 + (uintptr_t)yAlignedTo);
+        if (vec != 4 || !choose_line_args(g, numActive, y, a, threads, ld, lds, grid)) return 0;
+        const int lpp = 1 << a.lppLog;
+        out[0] = threads; out[1] = (int32_t)lds; out[2] = a.P; out[3] = a.Pp; out[4] = a.psplit; out[5] = a.Ct;
+        out[6] = a.cchunks; out[7] = ((a.P + LINE_EXT) * lpp + threads - 1) / threads; out[8] = ld;
+        out[9] = RS - (a.psplit - 1) * a.P;
+        out[10] = lines_match<LinesFixed<27, 27, 128, 3, 512>>(a, threads, ld) ||
+                  lines_match<LinesFixed<27, 27, 128, 2, 512>>(a, threads, ld) ||
+                  lines_match<LinesFixed<18, 18, 64, 2, 512>>(a, threads, ld);
+        return 1;
+    }
+    TileArgs a;
+    if (RS < 4) return 0;
+    if (kind == 1 ? !make_tile_args(g, numActive, vec, a, threads, lds, grid, 32 * 1024)
+                  : !scatter_tile_args(g, numActive, vec, a, threads, lds, grid))
+        return 0;
+    const int lpp = 1 << a.lppLog;
+    out[0] = threads; out[1] = (int32_t)lds; out[2] = a.P; out[3] = a.Pp; out[4] = a.psplit; out[5] = a.Ct;
+    out[6] = a.cchunks;
+    // per thread: NHWC items and planar slots of a full tile
+    const int items = (a.P * lpp + threads - 1) / threads;
+    const int slots = (int)((a.Ct * a.vpr + threads - 1) / threads);
+    out[7] = items > slots || kind == 1 ? items : slots;   // the gather's planar side loops, only its NHWC side is bounded
+    out[8] = TILE_LD;
+    out[9] = RS - (a.psplit - 1) * a.P;
+    out[10] = kind == 2 && vec == 4 &&
+              (tile_match<TileFixed<27, 27, 128, 124, 512>>(a, threads) || tile_match<TileFixed<27, 27, 128, 184, 512>>(a, threads) ||
+               tile_match<TileFixed<16, 16, 64, 128, 512>>(a, threads));
+    return 1;
+}
+
 hipError_t launch_gather(const float* x, float* y, const int16_t* idx, int numActive, const Geom& g,
                          bool transpose, hipStream_t stream)
 {

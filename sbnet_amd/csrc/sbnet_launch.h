@@ -45,6 +45,9 @@ hipError_t launch_reduce_mask(const float* mask, const Geom& g, int bCntH, int b
 constexpr size_t STATIC_SCRATCH_BYTES = (size_t)2 << 20;
 hipError_t static_scratch(void** ptr);
 
+// Test hook: see tile_choice in sbnet_kernels.hip.
+int tile_choice(int kind, const Geom& g, int numActive, int vec, int yAlignedTo, int32_t* out);
+
 hipError_t launch_gather(const float* x, float* y, const int16_t* idx, int numActive,
                          const Geom& g, bool transpose, hipStream_t stream);
 
