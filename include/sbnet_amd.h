@@ -211,9 +211,11 @@ size_t sbnet_sparse_scatter_workspace_bytes(int32_t num_active, const int64_t* y
  *   the overlapping values are equal.
  *   workspace   optional device scratch (4-byte aligned) of sbnet_sparse_scatter_workspace_bytes() bytes,
  *               or NULL.  Three uses.
- *               (0) add=0 and bstride < bsize: an owner map (one int32 per pixel: the last listed block that
- *               covers it) is built first and every block writes only the pixels it owns: the CPU functor's
- *               result, no pixel written twice.
+ *               (0) add=0 and bstride < bsize: every block writes only the pixels that no block listed later
+ *               covers: the CPU functor's result, no pixel written twice.  Which pixels those are comes from one
+ *               small extra launch that compares the blocks of the list pairwise (at most 2x2 blocks over a
+ *               pixel, bsize <= 2*bstride, and at most 4096 blocks; in-place op), or else from an owner map (one
+ *               int32 per pixel: the last listed block that covers it) built by two extra launches.
  *               (1) sbnet_sparse_scatter with atomic=0: when the blocks cover 16 MB or more, y is built from
  *               two disjoint parts instead of "copy ybase, scatter on top": pixels that no active block covers
  *               are copied from ybase, covered ones are written by the scatter, which reads ybase where it

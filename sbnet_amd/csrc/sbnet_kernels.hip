@@ -185,11 +185,35 @@ constexpr int SCATTER_COLOR = 3;  // kernel-side mode; callers ask for SCATTER_A
 // and a block listed twice is handled like any other overlap.
 constexpr int SCATTER_OWNED = 4;  // kernel-side mode; callers ask for SCATTER_ASSIGN and give scratch
 
+// The same order without a per-pixel map, for the common case of at most 2x2 blocks over a pixel (bsize <= 2 *
+// bstride) and a list short enough to compare every pair of blocks: a block's eight grid neighbours (and any other
+// row of the list that names the block itself) are the only blocks that can share pixels with it, and which of
+// its pixels a neighbour covers depends only on whether the pixel lies in the block's first R - U rows (shared
+// with the row of blocks above), its rows from U on (shared with the row below), or in between, and likewise for
+// columns.  k_rank_table leaves nine bits per block: bit 3*rowClass + colClass is set when some block listed
+// later covers that class of pixels; the scatter kernels skip those pixels.
+constexpr int SCATTER_RANKED = 5;  // kernel-side mode; callers ask for SCATTER_ASSIGN and give scratch
+
 struct ColorArgs {
     int kh, kw, pass;
     const int32_t* dup;
     const int32_t* owner;  // SCATTER_OWNED: [N, H, W] list positions, -1 where no block covers the pixel
+    const int32_t* rank;   // SCATTER_RANKED: nine bits per block, see k_rank_table
 };
+
+// Pixel (r, s) of a block against the block's nine bits: true when a block listed later covers it.
+__device__ __forceinline__ bool ranked_out(uint32_t bits, uint32_t r, uint32_t s, const Geom& g)
+{
+    const uint32_t rc = (int)r < g.R - g.U ? 0u : ((int)r >= g.U ? 2u : 1u);
+    const uint32_t cc = (int)s < g.S - g.V ? 0u : ((int)s >= g.V ? 2u : 1u);
+    return (bits >> (rc * 3u + cc)) & 1u;
+}
+
+__device__ __forceinline__ uint32_t rank_bits(const ColorArgs& col, uint32_t ib)
+{
+    typedef const int32_t __attribute__((address_space(4))) * const_i32_ptr;  // ib is wave-uniform: scalar load
+    return (uint32_t)*(const_i32_ptr)(reinterpret_cast<uintptr_t>(col.rank + ib));
+}
 
 // True when this launch has nothing to do for the block; `atomics` tells how to add otherwise.
 __device__ __forceinline__ bool color_skip(const ColorArgs& col, const BlockOrigin& o, bool& atomics)
@@ -308,6 +332,8 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc_wide(const float* __restri
                 if (MODE == SCATTER_OWNED &&
                     col.owner[((int64_t)o.n * a.g.H + hh) * a.g.W + o.w0 + (int)fdiv((uint32_t)j, a.dCV)] != (int32_t)ib)
                     dst[u] = -1;
+                else if (MODE == SCATTER_RANKED && ranked_out(rank_bits(col, ib), r, fdiv((uint32_t)j, a.dCV), a.g))
+                    dst[u] = -1;
                 else
                     v[u] = ld_stream(xb + e);
             }
@@ -321,7 +347,7 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc_wide(const float* __restri
 #pragma unroll
         for (int u = 0; u < NHWC_UNR; ++u)
             if (dst[u] >= 0) st_stream(yv + dst[u], vadd(cur[u], v[u]));
-    } else if (MODE == SCATTER_ASSIGN || MODE == SCATTER_OWNED) {
+    } else if (MODE == SCATTER_ASSIGN || MODE == SCATTER_OWNED || MODE == SCATTER_RANKED) {
 #pragma unroll
         for (int u = 0; u < NHWC_UNR; ++u)
             if (dst[u] >= 0) commit<VEC, SCATTER_ASSIGN>(yv + dst[u], v[u]);
@@ -591,7 +617,8 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
         const uint32_t r = fdiv(e, a.dRow);
         const int j = (int)(e - r * a.rowV);
         const int hh = o.h0 + (int)r;
-        const bool ok = e < a.blockV && (unsigned)hh < (unsigned)a.g.H && j >= lo && j < hi;
+        bool ok = e < a.blockV && (unsigned)hh < (unsigned)a.g.H && j >= lo && j < hi;
+        if (MODE == SCATTER_RANKED) ok = ok && !ranked_out(rank_bits(col, ib), r, fdiv((uint32_t)j, a.dCV), a.g);
         dst[u] = ok ? (((uint32_t)hh * (uint32_t)a.g.W + (uint32_t)o.w0) * (uint32_t)CV + (uint32_t)j) * (uint32_t)(VEC * 4)
                     : BUF_OOB;
         v[u] = buf_load<VEC>(xr, ok ? e * (uint32_t)(VEC * 4) : BUF_OOB);  // off-image parts are not read
@@ -604,7 +631,7 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
         // (an out-of-range owner read returns 0, which may equal ib: dst is BUF_OOB there already)
 #pragma unroll
         for (int u = 0; u < NHWC_UNR; ++u) buf_store<BUF_NT>(yr, own[u] == (int32_t)ib ? dst[u] : BUF_OOB, v[u]);
-    } else if (MODE == SCATTER_ASSIGN) {
+    } else if (MODE == SCATTER_ASSIGN || MODE == SCATTER_RANKED) {
 #pragma unroll
         for (int u = 0; u < NHWC_UNR; ++u) buf_store<BUF_NT>(yr, dst[u], v[u]);
     } else if (MODE == SCATTER_ADD || (MODE == SCATTER_COLOR && !atomics)) {
@@ -627,8 +654,8 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
 
 // NHWC side of a tile: thread tid owns channel vector cl = tid & (lpp-1) of pixels pl0 + u*step,
 // u = 0 .. TILE_LD-1, pl0 = tid >> lppLog, step = nthr >> lppLog.  Walks those pixels keeping (r, s) by
-// increments and hands each one's byte offset inside the image (or BUF_OOB) and its pixel number h*W + w (only
-// meaningful with an in-range offset) to `f(u, pl, off, pix)`.
+// increments and hands each one's byte offset inside the image (or BUF_OOB), its pixel number h*W + w (only
+// meaningful with an in-range offset) and its position (r, s) inside the block to `f(u, pl, off, pix, r, s)`.
 template <int VEC, typename G, typename F>
 __device__ __forceinline__ void nhwc_walk(const TileArgs& a, const TileId& t, const BlockOrigin& o, uint32_t tid,
                                           uint32_t nthr, F f)
@@ -647,7 +674,7 @@ __device__ __forceinline__ void nhwc_walk(const TileArgs& a, const TileId& t, co
         const int hh = o.h0 + (int)r, ww = o.w0 + (int)s;
         const bool ok = cok && pl < (uint32_t)t.Pn && (unsigned)hh < (unsigned)a.g.H && (unsigned)ww < (unsigned)a.g.W;
         const uint32_t off = (((uint32_t)hh * (uint32_t)a.g.W + (uint32_t)ww) * C + c) * 4u;
-        f(u, pl, ok ? off : BUF_OOB, (uint32_t)hh * (uint32_t)a.g.W + (uint32_t)ww);
+        f(u, pl, ok ? off : BUF_OOB, (uint32_t)hh * (uint32_t)a.g.W + (uint32_t)ww, r, s);
         pl += step;
         r += stepR;
         s += stepS;
@@ -677,7 +704,7 @@ __device__ __forceinline__ void gather_planar_tile(const float* __restrict__ x, 
 
     vec v[TILE_LD];
     uint32_t pls[TILE_LD];
-    nhwc_walk<VEC, TileRt>(a, t, o, tid, nthr, [&](int u, uint32_t pl, uint32_t off, uint32_t) {
+    nhwc_walk<VEC, TileRt>(a, t, o, tid, nthr, [&](int u, uint32_t pl, uint32_t off, uint32_t, uint32_t, uint32_t) {
         v[u] = buf_load<VEC>(xr, off);
         pls[u] = pl;
     });
@@ -1100,7 +1127,9 @@ __device__ __forceinline__ void scatter_planar_tile(const float* __restrict__ x,
     int32_t own[TILE_LD];
     const rsrc_t wr = make_rsrc(MODE == SCATTER_OWNED ? col.owner + (int64_t)o.n * a.g.H * a.g.W : nullptr,
                                 MODE == SCATTER_OWNED ? (uint32_t)(a.g.H * a.g.W) * 4u : 0u);
-    nhwc_walk<VEC, G>(a, t, o, tid, nthr, [&](int u, uint32_t pl, uint32_t off, uint32_t pix) {
+    const uint32_t rbits = MODE == SCATTER_RANKED ? rank_bits(col, t.ib) : 0u;
+    nhwc_walk<VEC, G>(a, t, o, tid, nthr, [&](int u, uint32_t pl, uint32_t off, uint32_t pix, uint32_t r, uint32_t sc) {
+        if (MODE == SCATTER_RANKED && ranked_out(rbits, r, sc, a.g)) off = BUF_OOB;
         offs[u] = off;
         if (MODE == SCATTER_OWNED) own[u] = __builtin_bit_cast(int32_t, buf_load<1>(wr, off != BUF_OOB ? pix * 4u : BUF_OOB));
         w[u] = vzero<VEC>();
@@ -1115,7 +1144,7 @@ __device__ __forceinline__ void scatter_planar_tile(const float* __restrict__ x,
     if (MODE == SCATTER_OWNED) {
 #pragma unroll
         for (int u = 0; u < TILE_LD; ++u) buf_store<BUF_NT>(yr, own[u] == (int32_t)t.ib ? offs[u] : BUF_OOB, w[u]);
-    } else if (MODE == SCATTER_ASSIGN) {
+    } else if (MODE == SCATTER_ASSIGN || MODE == SCATTER_RANKED) {
 #pragma unroll
         for (int u = 0; u < TILE_LD; ++u) buf_store<BUF_NT>(yr, offs[u], w[u]);
     } else if (MODE == SCATTER_ADD || (MODE == SCATTER_COLOR && !atomics)) {
@@ -1171,6 +1200,8 @@ __global__ __launch_bounds__(256) void k_planar_small(const float* __restrict__ 
         } else if (in) {
             if (MODE == SCATTER_OWNED) {
                 if (owner[((int64_t)o.n * g.H + hh) * g.W + ww] == (int32_t)ib) y[pix] = x[st];
+            } else if (MODE == SCATTER_RANKED) {
+                if (!ranked_out((uint32_t)owner[ib], (uint32_t)r, (uint32_t)s, g)) y[pix] = x[st];
             } else if (MODE == SCATTER_ASSIGN) y[pix] = x[st];
             else if (MODE == SCATTER_ADD) y[pix] = ysrc[pix] + x[st];
             else atomic_add_f32(y + pix, x[st]);
@@ -2021,7 +2052,7 @@ template <int VEC, int MODE>
 static bool launch_fixed_scatter(const float* x, float* y, const float* ysrc, const int16_t* idx, const TileArgs& a,
                                  int threads, size_t lds, int numActive, const ColorArgs& aux, hipStream_t stream)
 {
-    if constexpr (VEC == 4 && (MODE == SCATTER_ASSIGN || MODE == SCATTER_ADD)) {
+    if constexpr (VEC == 4 && (MODE == SCATTER_ASSIGN || MODE == SCATTER_ADD || MODE == SCATTER_RANKED)) {
         // 27x27 blocks of 128 channels with 16 KB and 24 KB tiles; 16x16 blocks of 64 channels
         return launch_fixed_scatter_one<VEC, MODE, TileFixed<27, 27, 128, 124, 512>>(x, y, ysrc, idx, a, threads, lds,
                                                                                       numActive, aux, stream) ||
@@ -2143,9 +2174,12 @@ hipError_t launch_gather(const float* x, float* y, const int16_t* idx, int numAc
 template <int VEC, int MODE>
 static void scatter_dispatch(const float* x, float* y, const float* ysrc, const int16_t* idx, const Geom& g,
                              int numActive, bool transpose, hipStream_t stream, hipError_t& err,
-                             const int32_t* owner = nullptr)
+                             const int32_t* order = nullptr)
 {
-    const ColorArgs aux{1, 1, 0, nullptr, owner};
+    // `order`: the owner map (SCATTER_OWNED) or the rank table (SCATTER_RANKED)
+    const ColorArgs aux{1, 1, 0, nullptr, MODE == SCATTER_OWNED ? order : nullptr,
+                        MODE == SCATTER_RANKED ? order : nullptr};
+    const int32_t* owner = order;
     if (!transpose) {
         NhwcArgs a;
         if (!make_nhwc_args(g, numActive, VEC, a)) { err = hipErrorInvalidValue; return; }
@@ -2176,10 +2210,13 @@ static void scatter_dispatch(const float* x, float* y, const float* ysrc, const 
 
 template <int VEC>
 static void scatter_mode(const float* x, float* y, const float* ysrc, const int16_t* idx, const Geom& g, int numActive,
-                         bool transpose, ScatterMode mode, hipStream_t stream, hipError_t& err, const int32_t* owner)
+                         bool transpose, ScatterMode mode, hipStream_t stream, hipError_t& err, const int32_t* order,
+                         bool ranked)
 {
-    if (mode == SCATTER_ASSIGN && owner)
-        scatter_dispatch<VEC, SCATTER_OWNED>(x, y, ysrc, idx, g, numActive, transpose, stream, err, owner);
+    if (mode == SCATTER_ASSIGN && order && ranked)
+        scatter_dispatch<VEC, SCATTER_RANKED>(x, y, ysrc, idx, g, numActive, transpose, stream, err, order);
+    else if (mode == SCATTER_ASSIGN && order)
+        scatter_dispatch<VEC, SCATTER_OWNED>(x, y, ysrc, idx, g, numActive, transpose, stream, err, order);
     else if (mode == SCATTER_ASSIGN)
         scatter_dispatch<VEC, SCATTER_ASSIGN>(x, y, ysrc, idx, g, numActive, transpose, stream, err);
     else if (mode == SCATTER_ADD)
@@ -2190,16 +2227,16 @@ static void scatter_mode(const float* x, float* y, const float* ysrc, const int1
 
 static hipError_t scatter_from(const float* x, float* y, const float* ysrc, const int16_t* idx, int numActive,
                                const Geom& g, bool transpose, ScatterMode mode, hipStream_t stream,
-                               const int32_t* owner = nullptr)
+                               const int32_t* order = nullptr, bool ranked = false)
 {
     if (numActive == 0) return hipSuccess;
     hipError_t err = hipSuccess;
     int vec = pick_vec(g, y, transpose ? nullptr : x);
     const int vsrc = pick_vec(g, ysrc, nullptr);
     if (vsrc < vec) vec = vsrc;
-    if (vec == 4) scatter_mode<4>(x, y, ysrc, idx, g, numActive, transpose, mode, stream, err, owner);
-    else if (vec == 2) scatter_mode<2>(x, y, ysrc, idx, g, numActive, transpose, mode, stream, err, owner);
-    else scatter_mode<1>(x, y, ysrc, idx, g, numActive, transpose, mode, stream, err, owner);
+    if (vec == 4) scatter_mode<4>(x, y, ysrc, idx, g, numActive, transpose, mode, stream, err, order, ranked);
+    else if (vec == 2) scatter_mode<2>(x, y, ysrc, idx, g, numActive, transpose, mode, stream, err, order, ranked);
+    else scatter_mode<1>(x, y, ysrc, idx, g, numActive, transpose, mode, stream, err, order, ranked);
     if (err != hipSuccess) return err;
     return hipGetLastError();
 }
@@ -2494,11 +2531,49 @@ static void make_cover_args(const Geom& g, int vec, CoverArgs& c)
     c.dS = make_fastdiv((uint32_t)g.S);
 }
 
+// Nine bits per block for SCATTER_RANKED.  One wave per block: the lanes compare the block with every row of the
+// list; a later row that names the same image and a grid position within one step in both directions sets the
+// classes of pixels it shares with the block (itself included: a block listed twice loses all its pixels to the
+// later row).
+constexpr int RANK_MAX_BLOCKS = 4096;   // rows compared pairwise: 16.8 M comparisons at most
+
+__global__ __launch_bounds__(256) void k_rank_table(const int16_t* __restrict__ idx, int numActive, Geom g,
+                                                    int32_t* __restrict__ table)
+{
+    const uint32_t lane = threadIdx.x & 63u;
+    const int ib = (int)(blockIdx.x * 4u + (threadIdx.x >> 6));
+    int count = numActive;
+    if (g.countDev) count = min(count, *g.countDev);
+    if (ib >= count) return;
+    const int n = idx[(size_t)ib * 3], bh = idx[(size_t)ib * 3 + 1], bw = idx[(size_t)ib * 3 + 2];
+    uint32_t bits = 0u;
+    for (int j = ib + 1 + (int)lane; j < count; j += 64) {
+        const int dn = idx[(size_t)j * 3] - n, dh = idx[(size_t)j * 3 + 1] - bh, dw = idx[(size_t)j * 3 + 2] - bw;
+        if (dn == 0 && dh >= -1 && dh <= 1 && dw >= -1 && dw <= 1) {
+            // row classes (0: first R-U rows, 1: middle, 2: rows from U on) that a block dh steps away covers
+            const uint32_t rows = dh < 0 ? 1u : (dh > 0 ? 4u : 7u), cols = dw < 0 ? 1u : (dw > 0 ? 4u : 7u);
+#pragma unroll
+            for (int rc = 0; rc < 3; ++rc)
+                if (rows & (1u << rc)) bits |= cols << (3 * rc);
+        }
+    }
+    for (int off = 32; off > 0; off >>= 1) bits |= (uint32_t)__shfl_xor((int)bits, off);
+    if (lane == 0) table[ib] = (int32_t)bits;
+}
+
+// The rank table applies when at most 2x2 blocks share a pixel and the list is short enough for pairwise comparison.
+static bool rank_table_applies(const Geom& g, int numActive)
+{
+    return numActive <= RANK_MAX_BLOCKS && g.R <= 2 * (int64_t)g.U && g.S <= 2 * (int64_t)g.V;
+}
+
 size_t scatter_owner_workspace_bytes(const Geom& g, int numActive)
 {
     if (numActive <= 0 || !(g.U < g.R || g.V < g.S)) return 0;  // only overlapping blocks need an order
     if ((int64_t)g.R * g.S >= (1ll << 31)) return 0;
-    return (size_t)g.N * g.H * g.W * 4 + 16;
+    // (the owner map; the rank table of the in-place op needs less, but the copying op always takes the map)
+    const size_t map = (size_t)g.N * g.H * g.W * 4 + 16, table = (size_t)numActive * 4 + 16;
+    return map > table ? map : table;
 }
 
 // Builds the owner map in `workspace`; false (nothing launched) when the ordered scatter does not apply.
@@ -2525,6 +2600,14 @@ hipError_t launch_scatter_owned(const float* x, float* y, const int16_t* idx, in
 {
     done = false;
     if (numActive == 0) { done = true; return hipSuccess; }
+    if (rank_table_applies(g, numActive) && scatter_owner_workspace_bytes(g, numActive) != 0 && workspace &&
+        workspaceBytes >= (size_t)numActive * 4 + 16 && (reinterpret_cast<uintptr_t>(workspace) & 3) == 0) {
+        int32_t* table = static_cast<int32_t*>(workspace);
+        hipLaunchKernelGGL(k_rank_table, dim3((unsigned)((numActive + 3) / 4)), dim3(256), 0, stream, idx, numActive, g,
+                           table);
+        done = true;
+        return scatter_from(x, y, y, idx, numActive, g, transpose, SCATTER_ASSIGN, stream, table, true);
+    }
     int32_t* owner = nullptr;
     if (!build_owner_map(idx, numActive, g, workspace, workspaceBytes, stream, owner)) return hipSuccess;
     done = true;
