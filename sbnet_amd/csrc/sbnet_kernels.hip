@@ -1496,13 +1496,22 @@ __global__ __launch_bounds__(256) void k_reduce_compact(const uint8_t* __restric
 // for the whole launch (still correct, to rounding).
 
 constexpr int PULL_NB_MAX = 9;   // (2*Kh - 1) * (2*Kw - 1) with Kh = ceil(R/U), Kw = ceil(S/V) <= 2
-constexpr int PULL_LOOP = 8;     // 64-vector steps per wave
+constexpr int PULL_STEPS = 3;    // 64-vector steps of one wave, all in flight together (1: 223 us, 2: 228, 3: 211, 4: 232
+                                 // on the 16x16-at-stride-8, 256-channel workload; 5 and more run out of registers)
+constexpr int PULL_CLASSES = 9;  // 3 row classes x 3 column classes of a block's pixels (see below)
+constexpr int PULL_COVER = 4;    // at most 2 x 2 blocks cover a pixel
+constexpr int PULL_TABLE_STRIDE = PULL_CLASSES * PULL_COVER * 2;  // ints per block
+
+// With at most 2x2 blocks over a pixel, which blocks cover a pixel of block (bh, bw) depends only on the pixel's
+// class: its row is among the first R-U rows (shared with the blocks one step up), among the rows from U on (one
+// step down) or in between (this row of blocks only), and the same for columns.  The table holds, per block and
+// class, the up to four active blocks that cover pixels of the class, sorted by list position, each as (position,
+// packed grid offset): the main kernel needs no search, and the first entry names the pixel's owner.
 
 struct PullArgs {
     Geom g;
     int bhMin, bwMin, nBH, nBW;  // extent of the inverse map: blocks that can touch the image
     int kh1, kw1;                // Kh - 1, Kw - 1
-    int tableStride;             // ints per block in the table: 1 + 2 * NB
     uint32_t CV, rowV, blockV;   // vectors per pixel, per block row, per block
     uint32_t cpb, units;         // wave-units per block, in total
     FastDiv dCpb, dRow, dCV;
@@ -1538,7 +1547,8 @@ __global__ __launch_bounds__(256) void k_pull_table(const int16_t* __restrict__ 
     const int ib = (int)(blockIdx.x * 256 + threadIdx.x);
     if (ib >= numActive || (a.g.countDev && ib >= *a.g.countDev)) return;
     const int n = idx[(size_t)ib * 3], bh = idx[(size_t)ib * 3 + 1], bw = idx[(size_t)ib * 3 + 2];
-    int ids[PULL_NB_MAX], offs[PULL_NB_MAX];
+    // the active blocks at most one step away (this one included), sorted by position in the list
+    int ids[PULL_NB_MAX], dhs[PULL_NB_MAX], dws[PULL_NB_MAX];
     int cnt = 0;
     if (pull_slot(a, n, bh, bw) >= 0) {
         for (int dh = -a.kh1; dh <= a.kh1; ++dh)
@@ -1546,22 +1556,37 @@ __global__ __launch_bounds__(256) void k_pull_table(const int16_t* __restrict__ 
                 const int64_t slot = pull_slot(a, n, bh + dh, bw + dw);
                 const int other = slot >= 0 ? map[slot] : -1;
                 if (other < 0) continue;
-                int k = cnt++;  // insertion sort by position in the active list
+                int k = cnt++;  // insertion sort
                 while (k > 0 && ids[k - 1] > other) {
                     ids[k] = ids[k - 1];
-                    offs[k] = offs[k - 1];
+                    dhs[k] = dhs[k - 1];
+                    dws[k] = dws[k - 1];
                     --k;
                 }
                 ids[k] = other;
-                offs[k] = ((dh & 0xffff) << 16) | (dw & 0xffff);
+                dhs[k] = dh;
+                dws[k] = dw;
             }
     }
-    int32_t* t = table + (size_t)ib * a.tableStride;
-    t[0] = cnt;
-    for (int k = 0; k < cnt; ++k) {
-        t[1 + 2 * k] = ids[k];
-        t[2 + 2 * k] = offs[k];
-    }
+    int32_t* t = table + (size_t)ib * PULL_TABLE_STRIDE;
+    for (int rc = 0; rc < 3; ++rc)
+        for (int cc = 0; cc < 3; ++cc) {
+            int m = 0;
+            for (int k = 0; k < cnt; ++k) {
+                // a block dh steps down covers row class 2 only, dh steps up class 0 only, the same row of blocks all
+                const bool rows = dhs[k] == 0 || (dhs[k] < 0 && rc == 0) || (dhs[k] > 0 && rc == 2);
+                const bool cols = dws[k] == 0 || (dws[k] < 0 && cc == 0) || (dws[k] > 0 && cc == 2);
+                if (rows && cols && m < PULL_COVER) {
+                    t[((rc * 3 + cc) * PULL_COVER + m) * 2] = ids[k];
+                    t[((rc * 3 + cc) * PULL_COVER + m) * 2 + 1] = ((dhs[k] & 0xffff) << 16) | (dws[k] & 0xffff);
+                    ++m;
+                }
+            }
+            for (; m < PULL_COVER; ++m) {
+                t[((rc * 3 + cc) * PULL_COVER + m) * 2] = -1;
+                t[((rc * 3 + cc) * PULL_COVER + m) * 2 + 1] = 0;
+            }
+        }
 }
 
 // sparse_gather.cc:103-130 with add == true on overlapping blocks, NHWC stack.
@@ -1583,60 +1608,77 @@ __global__ __launch_bounds__(256) void k_scatter_pull(const float* __restrict__ 
     if (!o.valid) return;
     const vec* __restrict__ xv = reinterpret_cast<const vec*>(x);
     vec* __restrict__ yv = reinterpret_cast<vec*>(y);
-    const bool atomicMode = *dup != 0;
-    const int32_t* __restrict__ t = table + (size_t)ib * a.tableStride;
-    const int cnt = atomicMode ? 0 : t[0];
-    int ids[PULL_NB_MAX], dhs[PULL_NB_MAX], dws[PULL_NB_MAX];
-#pragma unroll
-    for (int k = 0; k < PULL_NB_MAX; ++k) {
-        ids[k] = -1;
-        dhs[k] = 0;
-        dws[k] = 0;
-        if (k < cnt) {
-            ids[k] = t[1 + 2 * k];
-            const int packed = t[2 + 2 * k];
-            dhs[k] = (int)(int16_t)(packed >> 16) * a.g.U;
-            dws[k] = (int)(int16_t)(packed & 0xffff) * a.g.V;
+
+    if (*dup != 0) {
+        // the list names a block twice: the map cannot represent it; hardware atomics for the whole launch
+        for (int step = 0; step < PULL_STEPS; ++step) {
+            const uint32_t e = (chunk * PULL_STEPS + step) * 64 + lane;
+            if (e >= a.blockV) break;
+            const uint32_t r = fdiv(e, a.dRow);
+            const uint32_t j = e - r * a.rowV;
+            const uint32_t s = fdiv(j, a.dCV);
+            const int hh = o.h0 + (int)r, ww = o.w0 + (int)s;
+            if ((unsigned)hh >= (unsigned)a.g.H || (unsigned)ww >= (unsigned)a.g.W) continue;
+            vec* dst = yv + ((((int64_t)o.n * a.g.H + hh) * a.g.W + ww) * a.CV + (j - s * a.CV));
+            commit<VEC, SCATTER_ATOMIC>(dst, ld_stream(xv + ((size_t)ib * a.blockV + e)));
         }
+        return;
     }
 
-    for (int step = 0; step < PULL_LOOP; ++step) {
-        const uint32_t e = (chunk * PULL_LOOP + step) * 64 + lane;
-        if (e >= a.blockV) break;
+    // Phase 1: per vector, its class's table entries (two 16-byte loads from a table line that the whole block shares).
+    const int32_t* __restrict__ t = table + (size_t)ib * PULL_TABLE_STRIDE;
+    typedef int i4 __attribute__((ext_vector_type(4)));
+    i4 ent[PULL_STEPS][2];
+    uint32_t rr[PULL_STEPS], ss[PULL_STEPS], cvv[PULL_STEPS];
+    bool in[PULL_STEPS];
+#pragma unroll
+    for (int u = 0; u < PULL_STEPS; ++u) {
+        const uint32_t e = (chunk * PULL_STEPS + u) * 64 + lane;
         const uint32_t r = fdiv(e, a.dRow);
         const uint32_t j = e - r * a.rowV;
         const uint32_t s = fdiv(j, a.dCV);
-        const uint32_t cv = j - s * a.CV;
+        rr[u] = r;
+        ss[u] = s;
+        cvv[u] = j - s * a.CV;
         const int hh = o.h0 + (int)r, ww = o.w0 + (int)s;
-        if ((unsigned)hh >= (unsigned)a.g.H || (unsigned)ww >= (unsigned)a.g.W) continue;
-        vec* dst = yv + ((((int64_t)o.n * a.g.H + hh) * a.g.W + ww) * a.CV + cv);
-        if (atomicMode) {
-            commit<VEC, SCATTER_ATOMIC>(dst, ld_stream(xv + ((size_t)ib * a.blockV + e)));
-            continue;
+        in[u] = e < a.blockV && (unsigned)hh < (unsigned)a.g.H && (unsigned)ww < (unsigned)a.g.W;
+        const uint32_t rc = (int)r < a.g.R - a.g.U ? 0u : ((int)r >= a.g.U ? 2u : 1u);
+        const uint32_t cc = (int)s < a.g.S - a.g.V ? 0u : ((int)s >= a.g.V ? 2u : 1u);
+        const i4* q = reinterpret_cast<const i4*>(t + (in[u] ? (rc * 3u + cc) * (PULL_COVER * 2) : 0u));
+        ent[u][0] = q[0];
+        ent[u][1] = q[1];
+    }
+    // Phase 2: the owner of a pixel (the first of the blocks that cover it) reads the pixel and every contribution.
+    vec acc[PULL_STEPS], val[PULL_STEPS][PULL_COVER];
+    bool mine[PULL_STEPS], has[PULL_STEPS][PULL_COVER];
+    int64_t dstOff[PULL_STEPS];
+#pragma unroll
+    for (int u = 0; u < PULL_STEPS; ++u) {
+        const int id[PULL_COVER] = {ent[u][0].x, ent[u][0].z, ent[u][1].x, ent[u][1].z};
+        const int pk[PULL_COVER] = {ent[u][0].y, ent[u][0].w, ent[u][1].y, ent[u][1].w};
+        mine[u] = in[u] && id[0] == (int)ib;
+        const int hh = o.h0 + (int)rr[u], ww = o.w0 + (int)ss[u];
+        dstOff[u] = (((int64_t)o.n * a.g.H + hh) * a.g.W + ww) * a.CV + cvv[u];
+        // (loads under their own conditions: a load that no lane of the wave needs is skipped, and at one block
+        // in four active most pixels have one or two contributions, not four)
+        acc[u] = vzero<VEC>();
+        if (mine[u]) acc[u] = ld_stream(yv + dstOff[u]);
+#pragma unroll
+        for (int k = 0; k < PULL_COVER; ++k) {
+            has[u][k] = mine[u] && id[k] >= 0;
+            const int rs = (int)rr[u] - (int)(int16_t)(pk[k] >> 16) * a.g.U;
+            const int cs = (int)ss[u] - (int)(int16_t)(pk[k] & 0xffff) * a.g.V;
+            const int64_t off = (int64_t)id[k] * a.blockV + (int64_t)rs * a.rowV + (int64_t)cs * a.CV + cvv[u];
+            val[u][k] = vzero<VEC>();
+            if (has[u][k]) val[u][k] = ld_stream(xv + off);
         }
-        // which of the overlapping blocks cover this pixel, and is this block the first of them?
-        int64_t src[PULL_NB_MAX];
-        bool first = true, mine = false;
+    }
 #pragma unroll
-        for (int k = 0; k < PULL_NB_MAX; ++k) {
-            const int rr = (int)r - dhs[k], ss = (int)s - dws[k];
-            const bool covers = ids[k] >= 0 && (unsigned)rr < (unsigned)a.g.R && (unsigned)ss < (unsigned)a.g.S;
-            src[k] = covers ? ((int64_t)ids[k] * a.blockV + (int64_t)rr * a.rowV + (int64_t)ss * a.CV + cv) : -1;
-            if (covers && first) {
-                first = false;
-                mine = ids[k] == (int)ib;
-            }
-        }
-        if (!mine) continue;
-        vec acc = ld_stream(dst);
-        vec val[PULL_NB_MAX];
+    for (int u = 0; u < PULL_STEPS; ++u) {
 #pragma unroll
-        for (int k = 0; k < PULL_NB_MAX; ++k)
-            if (src[k] >= 0) val[k] = ld_stream(xv + src[k]);
-#pragma unroll
-        for (int k = 0; k < PULL_NB_MAX; ++k)
-            if (src[k] >= 0) acc = vadd(acc, val[k]);
-        st_stream(dst, acc);
+        for (int k = 0; k < PULL_COVER; ++k)
+            if (has[u][k]) acc[u] = vadd(acc[u], val[u][k]);  // ascending list position: the CPU functor's order
+        if (mine[u]) st_stream(yv + dstOff[u], acc[u]);
     }
 }
 
@@ -2270,17 +2312,16 @@ static bool make_map_args(const Geom& g, PullArgs& a, int64_t& mapN)
 static bool make_pull_args(const Geom& g, int numActive, int vec, PullArgs& a, int64_t& mapN)
 {
     const int Kh = (g.R + g.U - 1) / g.U, Kw = (g.S + g.V - 1) / g.V;
-    if ((2 * Kh - 1) * (2 * Kw - 1) > PULL_NB_MAX) return false;
+    if (Kh > 2 || Kw > 2) return false;  // at most 2x2 blocks over a pixel: neighbours one step away only
     if (!make_map_args(g, a, mapN)) return false;
     a.kh1 = Kh - 1;
     a.kw1 = Kw - 1;
-    a.tableStride = 1 + 2 * (2 * Kh - 1) * (2 * Kw - 1);
     const uint64_t rowV = (uint64_t)g.S * g.C / vec, blockV = rowV * g.R;
     if (blockV >= (1ull << 31)) return false;
     a.CV = (uint32_t)(g.C / vec);
     a.rowV = (uint32_t)rowV;
     a.blockV = (uint32_t)blockV;
-    a.cpb = (uint32_t)((blockV + 64 * PULL_LOOP - 1) / (64 * PULL_LOOP));
+    a.cpb = (uint32_t)((blockV + 64 * PULL_STEPS - 1) / (64 * PULL_STEPS));
     const uint64_t units = (uint64_t)numActive * a.cpb;
     if (units >= (1ull << 31)) return false;
     a.units = (uint32_t)units;
@@ -2295,7 +2336,7 @@ size_t scatter_pull_workspace_bytes(const Geom& g, int numActive)
     PullArgs a;
     int64_t mapN = 0;
     if (numActive <= 0 || !make_pull_args(g, numActive, 1, a, mapN)) return 0;
-    return (size_t)mapN * 4 + 16 + (size_t)numActive * a.tableStride * 4;
+    return (size_t)mapN * 4 + 16 + 16 + (size_t)numActive * PULL_TABLE_STRIDE * 4;  // map, flag, alignment, table
 }
 
 hipError_t launch_scatter_pull(const float* x, float* y, const int16_t* idx, int numActive, const Geom& g,
@@ -2311,7 +2352,8 @@ hipError_t launch_scatter_pull(const float* x, float* y, const int16_t* idx, int
         return hipSuccess;
     int32_t* map = static_cast<int32_t*>(workspace);
     int32_t* dup = map + mapN;
-    int32_t* table = dup + 4;
+    // the table is read with 16-byte loads
+    int32_t* table = reinterpret_cast<int32_t*>((reinterpret_cast<uintptr_t>(dup + 4) + 15) & ~(uintptr_t)15);
     int64_t fillWgs = (mapN + 255) / 256;
     if (fillWgs > 4096) fillWgs = 4096;
     if (fillWgs < 1) fillWgs = 1;
