@@ -1005,6 +1005,66 @@ def test_random_geometries(seed):
                 np.testing.assert_array_equal(host(y), y_o, err_msg=tag)
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_random_geometries_with_repeated_rows_and_device_counts(seed):
+    """The same kind of sweep with what the first one leaves out: lists that name blocks twice, counts that stay on
+    the device and stop short of the list, strides down to a third of the block (up to 3x3 blocks over a pixel),
+    and both the in-place and the copying op in every mode."""
+    for case in range(8):
+        rng = np.random.default_rng(50000 + 8 * seed + case)
+        N = int(rng.integers(1, 4))
+        C = int(rng.choice([1, 2, 3, 4, 6, 8, 12, 16, 20, 32, 36, 48, 64, 68, 128]))
+        R, S = int(rng.integers(1, 40)), int(rng.integers(1, 40))
+        U = int(rng.integers(max(1, R // 3), R + 3))
+        V = int(rng.integers(max(1, S // 3), S + 3))
+        H, W = int(rng.integers(R, 3 * R + 20)), int(rng.integers(S, 3 * S + 20))
+        bo = (int(rng.integers(-R + 1, 3)), int(rng.integers(-S + 1, 3)))
+        bc = bcount_covering(H, W, (U, V), bo)
+        cells = [(n, i, j) for n in range(N) for i in range(bc[0]) for j in range(bc[1]) if rng.random() < 0.6]
+        cells = sorted(set(cells + [(0, 0, 0), (N - 1, bc[0] - 1, bc[1] - 1)]))
+        dups = bool(rng.random() < 0.3)
+        if dups:
+            cells = cells + cells[:max(1, len(cells) // 5)]
+        idx = np.array(cells, np.int16)
+        rng.shuffle(idx, axis=0)
+        M = len(idx)
+        on_device = bool(rng.random() < 0.4)
+        Mc = int(rng.integers(1, M + 1)) if on_device else M
+        bin_counts = torch.tensor([Mc], dtype=torch.int32, device=DEV) if on_device else np.array([M], np.int32)
+        cnt_o = np.array([Mc], np.int32)
+        bs, bst = (R, S), (U, V)
+        tag = "seed %d case %d: N%d H%d W%d C%d bs %s bst %s bo %s M %d count %d repeats %s on device %s" % (
+            seed, case, N, H, W, C, bs, bst, bo, M, Mc, dups, on_device)
+        x = rng.integers(-8, 9, size=(N, H, W, C)).astype(np.float32)
+        base = rng.integers(-4, 5, size=(N, H, W, C)).astype(np.float32)
+        overlap = U < R or V < S
+        xd, idxd = dev(x), dev(idx)
+        for transpose in (False, True):
+            g_o = orc.sparse_gather(x, cnt_o, idx, bs, bst, bo, transpose=transpose)
+            shape = (M, C, R, S) if transpose else (M, R, S, C)
+            out = torch.full(shape, 7.0, device=DEV) if on_device else None
+            g = sbnet_amd.sparse_gather(xd, bin_counts, idxd, bs, bst, bo, transpose=transpose, out=out)
+            np.testing.assert_array_equal(host(g)[:Mc], g_o, err_msg=tag)
+            if on_device and Mc < M:
+                assert float(g[Mc:].min()) == 7.0 and float(g[Mc:].max()) == 7.0, tag   # rows past the count untouched
+            stack = rng.integers(-8, 9, size=shape).astype(np.float32)
+            sd = dev(stack)
+            modes = [(False, False), (True, True)] if (overlap or dups) else [(False, False), (True, False), (True, True)]
+            for add, atomic in modes:
+                if dups and not overlap and not add:
+                    continue   # repeated rows of tiling blocks, plain writes: the library orders overlapping geometries only
+                y_o = orc.sparse_scatter(stack[:Mc], cnt_o, idx, base, bs, bst, bo, add=add, atomic=atomic,
+                                         transpose=transpose)
+                what = tag + " add %s atomic %s transpose %s" % (add, atomic, transpose)
+                yv = dev(base)
+                sbnet_amd.sparse_scatter_var(sd, bin_counts, idxd, yv, bs, bst, bo, add=add, atomic=atomic,
+                                             transpose=transpose)
+                np.testing.assert_array_equal(host(yv), y_o, err_msg=what + " (in place)")
+                y = sbnet_amd.sparse_scatter(sd, bin_counts, idxd, dev(base), bs, bst, bo, add=add, atomic=atomic,
+                                             transpose=transpose)
+                np.testing.assert_array_equal(host(y), y_o, err_msg=what + " (copying)")
+
+
 # ---------------------------------------------------------------------------------------------
 # functor-level entry points and the copy
 # ---------------------------------------------------------------------------------------------
