@@ -1495,7 +1495,6 @@ __global__ __launch_bounds__(256) void k_reduce_compact(const uint8_t* __restric
 // be represented in the map; k_pull_map notices, and k_scatter_pull then falls back to hardware atomics
 // for the whole launch (still correct, to rounding).
 
-constexpr int PULL_NB_MAX = 9;   // (2*Kh - 1) * (2*Kw - 1) with Kh = ceil(R/U), Kw = ceil(S/V) <= 2
 constexpr int PULL_STEPS = 3;    // 64-vector steps of one wave, all in flight together (1: 223 us, 2: 228, 3: 211, 4: 232
                                  // on the 16x16-at-stride-8, 256-channel workload; 5 and more run out of registers)
 constexpr int PULL_CLASSES = 9;  // 3 row classes x 3 column classes of a block's pixels (see below)
@@ -1541,52 +1540,46 @@ __global__ __launch_bounds__(256) void k_pull_map(const int16_t* __restrict__ id
     if (atomicCAS(map + slot, -1, ib) != -1) *dup = 1;
 }
 
+// One thread per (block, class): the up to four active blocks that cover the class's pixels, sorted by position.
 __global__ __launch_bounds__(256) void k_pull_table(const int16_t* __restrict__ idx, int numActive, PullArgs a,
                                                     const int32_t* __restrict__ map, int32_t* __restrict__ table)
 {
-    const int ib = (int)(blockIdx.x * 256 + threadIdx.x);
+    const uint32_t t = blockIdx.x * 256u + threadIdx.x;
+    const int ib = (int)(t / PULL_CLASSES), cls = (int)(t % PULL_CLASSES);
     if (ib >= numActive || (a.g.countDev && ib >= *a.g.countDev)) return;
     const int n = idx[(size_t)ib * 3], bh = idx[(size_t)ib * 3 + 1], bw = idx[(size_t)ib * 3 + 2];
-    // the active blocks at most one step away (this one included), sorted by position in the list
-    int ids[PULL_NB_MAX], dhs[PULL_NB_MAX], dws[PULL_NB_MAX];
+    const int rc = cls / 3, cc = cls - rc * 3;
+    // a block one step up covers the first R-U rows only (row class 0), one step down the rows from U on (class 2)
+    const int dhLo = rc == 0 ? -a.kh1 : 0, dhHi = rc == 2 ? a.kh1 : 0;
+    const int dwLo = cc == 0 ? -a.kw1 : 0, dwHi = cc == 2 ? a.kw1 : 0;
+    int ids[PULL_COVER], pks[PULL_COVER];
     int cnt = 0;
     if (pull_slot(a, n, bh, bw) >= 0) {
-        for (int dh = -a.kh1; dh <= a.kh1; ++dh)
-            for (int dw = -a.kw1; dw <= a.kw1; ++dw) {
+        for (int dh = dhLo; dh <= dhHi; ++dh)
+            for (int dw = dwLo; dw <= dwHi; ++dw) {
                 const int64_t slot = pull_slot(a, n, bh + dh, bw + dw);
                 const int other = slot >= 0 ? map[slot] : -1;
                 if (other < 0) continue;
                 int k = cnt++;  // insertion sort
                 while (k > 0 && ids[k - 1] > other) {
                     ids[k] = ids[k - 1];
-                    dhs[k] = dhs[k - 1];
-                    dws[k] = dws[k - 1];
+                    pks[k] = pks[k - 1];
                     --k;
                 }
                 ids[k] = other;
-                dhs[k] = dh;
-                dws[k] = dw;
+                pks[k] = ((dh & 0xffff) << 16) | (dw & 0xffff);
             }
     }
-    int32_t* t = table + (size_t)ib * PULL_TABLE_STRIDE;
-    for (int rc = 0; rc < 3; ++rc)
-        for (int cc = 0; cc < 3; ++cc) {
-            int m = 0;
-            for (int k = 0; k < cnt; ++k) {
-                // a block dh steps down covers row class 2 only, dh steps up class 0 only, the same row of blocks all
-                const bool rows = dhs[k] == 0 || (dhs[k] < 0 && rc == 0) || (dhs[k] > 0 && rc == 2);
-                const bool cols = dws[k] == 0 || (dws[k] < 0 && cc == 0) || (dws[k] > 0 && cc == 2);
-                if (rows && cols && m < PULL_COVER) {
-                    t[((rc * 3 + cc) * PULL_COVER + m) * 2] = ids[k];
-                    t[((rc * 3 + cc) * PULL_COVER + m) * 2 + 1] = ((dhs[k] & 0xffff) << 16) | (dws[k] & 0xffff);
-                    ++m;
-                }
-            }
-            for (; m < PULL_COVER; ++m) {
-                t[((rc * 3 + cc) * PULL_COVER + m) * 2] = -1;
-                t[((rc * 3 + cc) * PULL_COVER + m) * 2 + 1] = 0;
-            }
-        }
+    typedef int i4 __attribute__((ext_vector_type(4)));
+    int e[PULL_COVER * 2];
+#pragma unroll
+    for (int k = 0; k < PULL_COVER; ++k) {
+        e[2 * k] = k < cnt ? ids[k] : -1;
+        e[2 * k + 1] = k < cnt ? pks[k] : 0;
+    }
+    i4* q = reinterpret_cast<i4*>(table + (size_t)ib * PULL_TABLE_STRIDE + cls * (PULL_COVER * 2));
+    q[0] = (i4){e[0], e[1], e[2], e[3]};
+    q[1] = (i4){e[4], e[5], e[6], e[7]};
 }
 
 // sparse_gather.cc:103-130 with add == true on overlapping blocks, NHWC stack.
@@ -2360,7 +2353,8 @@ hipError_t launch_scatter_pull(const float* x, float* y, const int16_t* idx, int
     const unsigned perBlockWgs = (unsigned)((numActive + 255) / 256);
     hipLaunchKernelGGL(k_pull_fill, dim3((unsigned)fillWgs), dim3(256), 0, stream, map, mapN, dup);
     hipLaunchKernelGGL(k_pull_map, dim3(perBlockWgs), dim3(256), 0, stream, idx, numActive, a, map, dup);
-    hipLaunchKernelGGL(k_pull_table, dim3(perBlockWgs), dim3(256), 0, stream, idx, numActive, a, map, table);
+    hipLaunchKernelGGL(k_pull_table, dim3((unsigned)(((int64_t)numActive * PULL_CLASSES + 255) / 256)), dim3(256), 0,
+                       stream, idx, numActive, a, map, table);
     const unsigned wgs = (a.units + 3) / 4;
     if (vec == 4) hipLaunchKernelGGL(k_scatter_pull<4>, dim3(wgs), dim3(256), 0, stream, x, y, idx, a, table, dup);
     else if (vec == 2) hipLaunchKernelGGL(k_scatter_pull<2>, dim3(wgs), dim3(256), 0, stream, x, y, idx, a, table, dup);
