@@ -1932,11 +1932,12 @@ static int device_cus()
 // 9.08 -> 8.87 us at 58 blocks, 20.6 -> 19.9 us at 156, but 40.8 -> 41.4 us at 312).
 constexpr int SCATTER_FEW_WGS_PER_CU = 22;
 
+// `share`: the launch does work for one block in `share` only (the passes of an overlapping add).
 static bool scatter_tile_args(const Geom& g, int numActive, int vec, TileArgs& a, int& threads, size_t& ldsBytes,
-                              unsigned& grid)
+                              unsigned& grid, int share = 1)
 {
     if (!make_tile_args(g, numActive, vec, a, threads, ldsBytes, grid, 16 * 1024)) return false;
-    if (a.psplit > 1 && a.total < (uint32_t)(SCATTER_FEW_WGS_PER_CU * device_cus())) {
+    if (a.psplit > 1 && a.total / (uint32_t)share < (uint32_t)(SCATTER_FEW_WGS_PER_CU * device_cus())) {
         TileArgs b;
         int bt;
         size_t bl;
@@ -2397,7 +2398,7 @@ static bool color_passes(const float* x, float* y, const int16_t* idx, const Geo
         int threads;
         size_t lds;
         unsigned grid;
-        if ((int64_t)g.R * g.S < 4 || !scatter_tile_args(g, numActive, VEC, a, threads, lds, grid)) return false;
+        if ((int64_t)g.R * g.S < 4 || !scatter_tile_args(g, numActive, VEC, a, threads, lds, grid, passes)) return false;
         for (col.pass = 0; col.pass < passes; ++col.pass)
             hipLaunchKernelGGL((k_scatter_planar<VEC, SCATTER_COLOR, TileRt>), tile_grid(a.grid2d, a.tpb, numActive, a.total, a.g),
                                dim3(threads), lds, stream, x, y, (const float*)y, idx, a, col);
@@ -2433,7 +2434,7 @@ hipError_t launch_scatter_colored(const float* x, float* y, const int16_t* idx, 
         size_t lds;
         unsigned grid;
         if (!transpose ? !make_nhwc_args(g, numActive, vec, na)
-                       : ((int64_t)g.R * g.S < 4 || !scatter_tile_args(g, numActive, vec, ta, threads, lds, grid)))
+                       : ((int64_t)g.R * g.S < 4 || !scatter_tile_args(g, numActive, vec, ta, threads, lds, grid, col.kh * col.kw)))
             return hipSuccess;
     }
     int64_t fillWgs = (mapN + 255) / 256;
