@@ -584,8 +584,8 @@ void* sbnet_scratch_acquire(size_t bytes, void* stream)
     // growing allocates, which a stream under capture must not do
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(s, &cap) != hipSuccess) {
-        (void)hipGetLastError();
-        return nullptr;
+        (void)hipGetLastError();  // a stream that cannot be asked is not being captured
+        cap = hipStreamCaptureStatusNone;
     }
     if (cap != hipStreamCaptureStatusNone) return nullptr;
     size_t want = (size_t)1 << 20;
