@@ -1266,8 +1266,9 @@ __device__ __forceinline__ void publish_count(int total, int fixupZero, int16_t*
         total = 1;
     }
     *binCount = total;
+    // (relaxed: the host takes nothing but this word from the device; a release here would first write back the L2)
     if (hostSignal)
-        __hip_atomic_store(hostSignal, ((unsigned long long)hostSeq << 32) | (uint32_t)total, __ATOMIC_RELEASE,
+        __hip_atomic_store(hostSignal, ((unsigned long long)hostSeq << 32) | (uint32_t)total, __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
