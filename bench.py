@@ -61,6 +61,9 @@ def parse():
     ap.add_argument("--ops-only", action="store_true",
                     help="per-op tables only (ops_by_density), no pipeline timing: a kernel trace of this run holds "
                          "exactly the launches the per-op times and the roofline come from")
+    ap.add_argument("--kernel-digest", action="store_true",
+                    help="print the digest of the kernel sources (the `kernel_source_sha256=` line a counter summary "
+                         "under profiles/ carries) and exit")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run the library's plain copy kernel on 256 MiB, 10 times: a kernel of known traffic "
                          "against which profiler byte counters are scaled")
@@ -368,24 +371,50 @@ def cpu_baseline(wl, M, idx_host, nbytes, budget_s=12.0):
              "ms_per_pass": round(tm * 1e3, 2)})
 
 
+def kernel_source_digest():
+    """sha256 over the device sources the library is built from (csrc/*.hip and csrc/*.h, by name): the counters
+    under profiles/ belong to one state of them."""
+    import glob
+    import hashlib
+    d = os.path.join(ROOT, "sbnet_amd", "csrc")
+    h = hashlib.sha256()
+    for p in sorted(glob.glob(os.path.join(d, "*.hip")) + glob.glob(os.path.join(d, "*.h"))):
+        h.update(os.path.basename(p).encode() + b"\0")
+        with open(p, "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
 def read_measured_traffic(name, op):
     """HBM bytes per launch of `op` ("gather" or "scatter") measured with rocprofv3 --pmc, if a summary under
-    profiles/ records them as lines `<op>_fetch_bytes_per_launch=<int>` and `<op>_write_bytes_per_launch=<int>`."""
+    profiles/ records them as lines `<op>_fetch_bytes_per_launch=<int>` and `<op>_write_bytes_per_launch=<int>`.
+    Returns (bytes, note).  The summary names the kernel source it was measured on (`kernel_source_sha256=`); when
+    the source has changed since, the counters no longer describe these kernels and the bytes are None."""
     p = os.path.join(ROOT, "profiles", name)
     if not os.path.exists(p):
-        return None
-    vals = {}
+        return None, "no counter summary under profiles/"
+    vals, digest = {}, None
     for line in open(p):
+        line = line.strip()
+        if line.startswith("kernel_source_sha256="):
+            digest = line.split("=", 1)[1].split()[0]
         for key in ("%s_fetch_bytes_per_launch" % op, "%s_write_bytes_per_launch" % op):
-            if line.strip().startswith(key + "="):
+            if line.startswith(key + "="):
                 vals[key] = int(float(line.split("=", 1)[1].split()[0]))
-    if len(vals) == 2:
-        return sum(vals.values())
-    return None
+    if len(vals) != 2:
+        return None, "profiles/%s holds no counters for the %s" % (name, op)
+    if digest != kernel_source_digest():
+        return None, ("profiles/%s was measured on another state of the kernel sources: its counters are stale "
+                      "until its commands are run again" % name)
+    return sum(vals.values()), ("profiles/%s (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by the copy kernel, on "
+                                "this kernel source; not re-measured by this run)" % name)
 
 
 def main():
     args = parse()
+    if args.kernel_digest:
+        print(kernel_source_digest())
+        return
     if args.gpus != 1:
         print("bench.py: this path is measured on one GPU only (one MI355X per box); --gpus %d is not supported. "
               "The path shards by image (n) with no exchange between GPUs." % args.gpus, file=sys.stderr)
@@ -510,14 +539,15 @@ def main():
     kernel_names = {"gather": "planar gather of sparse_gather(transpose=True): k_gather_lines",
                     "scatter": "planar scatter of sparse_scatter_var(add=False, transpose=True): k_scatter_planar"}
     traffic_file = "gather_lines_scatter_planar_C3_30pct_pmc.txt"
-    traffic = read_measured_traffic(traffic_file, dom) if round(args.density * 100) == 30 else None
+    if round(args.density * 100) == 30:
+        traffic, traffic_note = read_measured_traffic(traffic_file, dom)
+    else:
+        traffic, traffic_note = None, "counters were collected at 30 % density only"
     roofline = {"bound": "hbm", "kernel": kernel_names[dom],
                 "achieved": g["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(g["GBps"] / HBM_PEAK_GBS, 4), "us_per_launch": g["us"],
                 "algorithmic_bytes_per_launch": g["bytes"],
-                "traffic": traffic,
-                "traffic_source": ("profiles/%s (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by the copy kernel; "
-                                   "not re-measured by this run)" % traffic_file) if traffic else None}
+                "traffic": traffic, "traffic_source": traffic_note}
     if traffic:
         # the same launch time against the bytes the profiler counted between L2 and the fabric
         roofline["traffic_GBps"] = round(traffic / g["us"] * 1e-3, 1)
