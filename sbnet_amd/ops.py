@@ -146,6 +146,30 @@ def reduce_mask(mask, dynamic_bcount, dynamic_bsize, dynamic_bstride, dynamic_bo
     return ReduceMaskResult(idx, dev_count)
 
 
+def reduce_mask_functor(mask, bcount, bsize, bstride, boffset, tol, avgpool=False):
+    """ReduceMaskFunctor (reduce_mask.h:23-44): the op without its host read-back and without the "no active block"
+    fix-up of ReduceMaskOp::Compute (reduce_mask.cc:206-218).  Returns (active_block_indices, count): the int16
+    list as reduce_mask returns it and an int32 GPU tensor [1] with the raw count, which can be 0.  Does not wait."""
+    lib = _lib.load()
+    mask = _dev_f32(mask, "mask")
+    if mask.dim() not in (3, 4) or (mask.dim() == 4 and mask.shape[3] != 1):
+        raise InvalidArgument("mask must be [N,H,W,1] (or [N,H,W]), got %s" % (tuple(mask.shape),))
+    N, H, W = int(mask.shape[0]), int(mask.shape[1]), int(mask.shape[2])
+    (bc, bcp, bcl), (bs, _, bsl), (bt, _, btl), (bo, _, bol) = _pair(bcount), _pair(bsize), _pair(bstride), _pair(boffset)
+    if not (bcl == bsl == btl == bol == 2):
+        _check(_lib.SBNET_EINVAL_PARAM_SHAPE)
+    with torch.cuda.device(mask.device):
+        max_idx = lib.sbnet_reduce_mask_max_indices(N, bcp, bcl)
+        idx = torch.empty((max(int(max_idx), 1), 3), dtype=torch.int16, device=mask.device)
+        ws = _workspace(mask.device, lib.sbnet_reduce_mask_workspace_bytes(N, bcp, bcl))
+        count = torch.empty(1, dtype=torch.int32, device=mask.device)
+        _check(lib.sbnet_reduce_mask_functor(mask.data_ptr(), N, H, W, ctypes.c_float(tol), int(bo[0]), int(bo[1]),
+                                             int(bs[0]), int(bs[1]), int(bt[0]), int(bt[1]), int(bc[0]), int(bc[1]),
+                                             1, 1, idx.data_ptr(), count.data_ptr(), int(bool(avgpool)),
+                                             ws.data_ptr(), ws.numel(), _stream()))
+    return idx, count
+
+
 def sparse_gather(x, bin_counts, active_block_indices, dynamic_bsize, dynamic_bstride, dynamic_boffset,
                   transpose=False, out=None):
     """SparseGather (sparse_gather.cc:48-57, 160-218): x [N,H,W,C] -> [M,bsize[0],bsize[1],C], or

@@ -3,7 +3,10 @@
 Mirrors the user-facing layer functions of the reference's model library,
 sbnet_tensorflow/benchmark/sparse_conv_lib.py: `convert_mask_to_indices_custom` (424-459),
 `sparse_conv2d_custom` (536-587), `_bottleneck_residual` (677-723), `res_block_bottleneck`
-(726-748), `sparse_res_block_bottleneck` (751-824) and `mask_conv2d` (891-911).  The three block ops
+(726-748), `sparse_res_block_bottleneck` (751-824) and `mask_conv2d` (891-911), and its index-list interface
+`convert_mask_to_indices` (279-318), `upsample_indices` (249-276), `convert_mask_to_block_indices` (321-340),
+`sparse_conv2d` (462-523) and `sparse_conv2d_matmul` (827-888), which the reference computes with TensorFlow's
+gather_nd / scatter_nd and which here run on the same block ops.  The three block ops
 run the HIP kernels of this package; the dense convolutions, batch norm and ReLU between gather and
 scatter are PyTorch's (MIOpen on this hardware), exactly where the reference calls cuDNN.
 
@@ -18,7 +21,7 @@ import collections
 import torch
 import torch.nn.functional as F
 
-from . import _lib, ops
+from . import _lib, block_params, ops
 
 BN_DECAY = 0.999   # tf.contrib.layers.batch_norm defaults used by the reference (sparse_conv_lib.py:600-601)
 BN_EPS = 0.001
@@ -73,6 +76,144 @@ def mask_conv2d(x, w, mask, strides, padding):
     y = _conv_same_or_valid(x.permute(0, 3, 1, 2), _hwio_to_oihw(w), (strides[1], strides[2]), padding)
     m = _pool_same_or_valid(mask.permute(0, 3, 1, 2), (kh, kw), (strides[1], strides[2]), padding)
     return (y * m).permute(0, 2, 3, 1).contiguous()
+
+
+# ---------------------------------------------------------------------------------------------
+# The reference's index-list interface (its TensorFlow-only twin of the custom ops): the same names and
+# argument meaning, computed with this package's block ops
+# ---------------------------------------------------------------------------------------------
+
+def _pad_amounts(h, w, ksize, strides, padding, bsize=None, bstrides=None):
+    """(top, bottom, left, right) zero padding of sparse_conv_lib.py:150-189 (_pad_input): TensorFlow's SAME / VALID
+    padding, the far side extended so that the last block fits when block size and strides are given."""
+    ph0, ph1, pw0, pw1 = block_params.calc_padding_4d([1, h, w, 1], ksize, strides, padding)
+    if bstrides is not None:
+        assert bsize is not None, "Must pass in bsize and bstrides together."
+        ph1 += (-(h + ph0 + ph1) + bsize[1]) % bstrides[1]
+        pw1 += (-(w + pw0 + pw1) + bsize[2]) % bstrides[2]
+    return ph0, ph1, pw0, pw1
+
+
+def upsample_indices(indices, ksize, strides):
+    """sparse_conv_lib.py:249-276: block positions [M,3] (n, i, j) of a pooling with window `ksize` and step
+    `strides` -> [M, ksize[1], ksize[2], 3], the (n, h, w) of every pixel of each window.  int32."""
+    assert indices.dim() == 2, "Expect indices rank = 2"
+    assert ksize[0] == ksize[3] == 1, "Expect first and last dimensions of ksize = 1"
+    assert strides[0] == strides[3] == 1, "Expect first and last dimensions of strides = 1, {}".format(strides)
+    dev = indices.device
+    top_left = indices.to(torch.int32) * torch.tensor([1, strides[1], strides[2]], dtype=torch.int32, device=dev)
+    r = torch.arange(ksize[1], dtype=torch.int32, device=dev).view(1, -1, 1)
+    c = torch.arange(ksize[2], dtype=torch.int32, device=dev).view(1, 1, -1)
+    n = top_left[:, 0].view(-1, 1, 1).expand(-1, ksize[1], ksize[2])
+    h = top_left[:, 1].view(-1, 1, 1) + r
+    w = top_left[:, 2].view(-1, 1, 1) + c
+    return torch.stack([n, h.expand(-1, -1, ksize[2]), w.expand(-1, ksize[1], -1)], dim=3)
+
+
+def convert_mask_to_indices(mask, bsize, ksize, strides, padding, tol):
+    """sparse_conv_lib.py:279-318: mask [N,H,W] -> int32 [M,3], the (n, i, j) of the blocks whose maximum over the
+    zero-padded mask exceeds tol, in row-major order.  Runs reduce_mask's kernels (max pooling, ordered
+    compaction); the list is cut to its length on the host, as tf.where's dynamic shape is."""
+    assert mask.dim() == 3, "Expect mask rank = 3"
+    assert isinstance(bsize, (list, tuple)), "`bsize` needs to be a list or tuple."
+    assert isinstance(ksize, (list, tuple)), "`ksize` needs to be a list or tuple."
+    assert isinstance(strides, (list, tuple)), "`strides` needs to be a list or tuple."
+    err_div = "Expect `stride` divides `bsize` - `ksize`. stride {}, bsize {}, ksize {}."
+    assert (bsize[1] - ksize[0]) % strides[1] == 0, err_div.format(strides[1], bsize[1], ksize[0])
+    assert (bsize[2] - ksize[1]) % strides[2] == 0, err_div.format(strides[2], bsize[2], ksize[1])
+    assert strides[0] == strides[3] == 1, "Expect first and last dimensions of strides = 1. Dim {}.".format(strides)
+    bstrides = block_params.calc_block_strides(bsize, ksize, strides)
+    h, w = int(mask.shape[1]), int(mask.shape[2])
+    ph0, ph1, pw0, pw1 = _pad_amounts(h, w, ksize, strides, padding, bsize, bstrides)
+    bcount = [(h + ph0 + ph1 - bsize[1]) // bstrides[1] + 1, (w + pw0 + pw1 - bsize[2]) // bstrides[2] + 1]
+    if mask.shape[0] == 0 or bcount[0] <= 0 or bcount[1] <= 0:
+        return torch.zeros((0, 3), dtype=torch.int32, device=mask.device)
+    boffset = [-ph0, -pw0]
+    if tol < 0:
+        # padding zeros exceed a negative tol, pixels outside the image never do: pad for real
+        mask = F.pad(mask, (pw0, pw1, ph0, ph1))
+        boffset = [0, 0]
+    idx, count = ops.reduce_mask_functor(mask.contiguous(), bcount, bsize[1:3], bstrides[1:3], boffset, tol)
+    return idx[:int(count.item())].to(torch.int32)
+
+
+def convert_mask_to_block_indices(mask, bsize, ksize, strides, padding, tol):
+    """sparse_conv_lib.py:321-340: mask [N,H,W] -> int32 [M, bsize[1], bsize[2], 3], the pixels (in the padded
+    input's coordinates) of every active block."""
+    indices = convert_mask_to_indices(mask, bsize, ksize, strides, padding, tol)
+    return upsample_indices(indices, bsize, block_params.calc_block_strides(bsize, ksize, strides))
+
+
+def _rect_origins(blk_indices):
+    """int16 (n, h0, w0) rows of the rectangles of a [M,h,w,3] pixel-index tensor, for block ops that step by one
+    pixel: block (n, bh, bw) then starts at pixel (boffset + bh, boffset + bw)."""
+    assert blk_indices.dim() == 4 and blk_indices.shape[3] == 3, "Expect blk_indices of shape [M, h, w, 3]"
+    bh, bw = int(blk_indices.shape[1]), int(blk_indices.shape[2])
+    origin = blk_indices[:, 0, 0, :].to(torch.int32)
+    if blk_indices.shape[0]:
+        want = upsample_indices(origin, [1, bh, bw, 1], [1, 1, 1, 1])
+        if not bool((want == blk_indices.to(torch.int32)).all()):
+            raise ValueError("blk_indices must list the pixels of axis-aligned rectangles in row-major order")
+        lo, hi = int(origin.min()), int(origin.max())
+        if lo < 0 or hi > 32767:
+            raise ValueError("block positions must lie in [0, 32767]")
+    return origin.to(torch.int16).contiguous()
+
+
+def _scatter_rectangles(q, origins, count, out_shape):
+    """tf.scatter_nd of a stack of rectangles into zeros: q [M, qh, qw, K] lands with its top-left pixel at
+    origins[m] = (n, h, w); rectangles that meet are summed; pixels outside `out_shape` are dropped."""
+    y = torch.zeros(out_shape, dtype=torch.float32, device=q.device)
+    if q.shape[0] == 0:
+        return y
+    geom = ([int(q.shape[1]), int(q.shape[2])], [1, 1], [0, 0])
+    if torch.is_grad_enabled() and q.requires_grad:
+        return ops.sparse_scatter(q, count, origins, y, *geom, add=True, atomic=True)
+    return ops.sparse_scatter_var(q.contiguous(), count, origins, y, *geom, add=True, atomic=True)
+
+
+def sparse_conv2d(x, w, blk_indices, strides, padding):
+    """sparse_conv_lib.py:462-523: convolution evaluated on the rectangles of `blk_indices` only.
+
+    x [N,H,W,C]; w [kh,kw,C,K]; blk_indices int32 [M,h,w,3] as convert_mask_to_block_indices returns them
+    (pixels of M rectangles in the zero-padded input's coordinates).  Each rectangle is gathered (pixels of the
+    padding read as zeros, so the input is not padded in memory), convolved VALID with `strides`, and its result
+    is written at the rectangle's position in a zero tensor of the convolution's output shape [N,H',W',K]."""
+    ksize = [int(v) for v in w.shape]
+    out_shape = block_params.calc_out_size_4d([int(v) for v in x.shape], ksize, strides, padding)
+    origins = _rect_origins(blk_indices)
+    M, bh, bw = int(blk_indices.shape[0]), int(blk_indices.shape[1]), int(blk_indices.shape[2])
+    if M == 0:
+        return torch.zeros(out_shape, dtype=torch.float32, device=x.device)
+    ph0, _, pw0, _ = block_params.calc_padding_4d([int(v) for v in x.shape], ksize, strides, padding)
+    count = torch.tensor([M], dtype=torch.int32)
+    p = ops.sparse_gather(x, count, origins, [bh, bw], [1, 1], [-ph0, -pw0])
+    q = _conv_blocks(p, w, (strides[1], strides[2]), False)
+    # a rectangle at padded-input pixel (h0, w0) produces the outputs from (h0 // stride, w0 // stride) on
+    out_origins = origins.clone()
+    out_origins[:, 1] = torch.div(origins[:, 1], strides[1], rounding_mode="floor")
+    out_origins[:, 2] = torch.div(origins[:, 2], strides[2], rounding_mode="floor")
+    return _scatter_rectangles(q, out_origins, count, out_shape)
+
+
+def sparse_conv2d_matmul(x, w, blk_indices, strides, padding):
+    """sparse_conv_lib.py:827-888: the same for rectangles of exactly the kernel's size and stride 1: every
+    rectangle is one output pixel, computed as a matrix product of the gathered patches with the flattened kernel."""
+    ksize = [int(v) for v in w.shape]
+    if int(blk_indices.shape[1]) != ksize[0] or int(blk_indices.shape[2]) != ksize[1]:
+        raise ValueError("Expect blk_indices.shape[1] == w.shape[0] and blk_indices.shape[2] == w.shape[1].")
+    if strides[1] != 1 or strides[2] != 1:
+        raise ValueError("Strides > 1 not supported.")
+    out_shape = block_params.calc_out_size_4d([int(v) for v in x.shape], ksize, strides, padding)
+    origins = _rect_origins(blk_indices)
+    M = int(blk_indices.shape[0])
+    if M == 0:
+        return torch.zeros(out_shape, dtype=torch.float32, device=x.device)
+    ph0, _, pw0, _ = block_params.calc_padding_4d([int(v) for v in x.shape], ksize, strides, padding)
+    count = torch.tensor([M], dtype=torch.int32)
+    p = ops.sparse_gather(x, count, origins, [ksize[0], ksize[1]], [1, 1], [-ph0, -pw0])
+    q = p.reshape(M, ksize[0] * ksize[1] * ksize[2]) @ w.reshape(ksize[0] * ksize[1] * ksize[2], ksize[3])
+    return _scatter_rectangles(q.view(M, 1, 1, ksize[3]), origins, count, out_shape)
 
 
 def _same_pads(size, k, s):

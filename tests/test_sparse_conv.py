@@ -229,3 +229,176 @@ def test_sparse_res_block_in_a_hip_graph_replays_identically(data_format):
                                                  data_format=data_format)
             torch.cuda.synchronize()
             np.testing.assert_array_equal(got.cpu().numpy(), exp.cpu().numpy())
+
+
+# ---------------------------------------------------------------------------------------------
+# The reference's index-list interface (convert_mask_to_block_indices / upsample_indices / sparse_conv2d /
+# sparse_conv2d_matmul), pinned by the vectors its own tests hold
+# ---------------------------------------------------------------------------------------------
+
+# benchmark/sparse_conv_tests.py:68-100: two 3x3 windows at (0,1,2) and (0,2,0), stride 1
+UPSAMPLE_IND = [[0, 1, 2], [0, 2, 0]]
+UPSAMPLE_EXP = [[0, 1, 2], [0, 1, 3], [0, 1, 4], [0, 2, 2], [0, 2, 3], [0, 2, 4], [0, 3, 2], [0, 3, 3], [0, 3, 4],
+                [0, 2, 0], [0, 2, 1], [0, 2, 2], [0, 3, 0], [0, 3, 1], [0, 3, 2], [0, 4, 0], [0, 4, 1], [0, 4, 2]]
+
+
+def test_upsample_indices_known_answer():
+    from sbnet_amd import sparse_conv as sc
+    ind = torch.tensor(UPSAMPLE_IND, dtype=torch.int32, device=DEV)
+    up = sc.upsample_indices(ind, [1, 3, 3, 1], [1, 1, 1, 1])
+    assert tuple(up.shape) == (2, 3, 3, 3) and up.dtype == torch.int32
+    np.testing.assert_array_equal(up.cpu().numpy().reshape(-1, 3), np.asarray(UPSAMPLE_EXP, np.int32))
+    # a pooling step of 2 moves the windows, not their pixels (sparse_conv_lib.py:266-275)
+    up2 = sc.upsample_indices(ind, [1, 2, 3, 1], [1, 2, 2, 1]).cpu().numpy()
+    assert up2.shape == (2, 2, 3, 3)
+    np.testing.assert_array_equal(up2[0, :, :, 1:], [[[2, 4], [2, 5], [2, 6]], [[3, 4], [3, 5], [3, 6]]])
+
+
+@pytest.mark.parametrize("padding,y_exp", [
+    # benchmark/sparse_conv_tests.py:107-148 (VALID) and 150-193 (SAME): the same two hand-written rectangles
+    ("VALID", [[0, 0, 0], [0, 0, 9], [9, 0, 0]]),
+    ("SAME", [[0, 0, 0, 0, 0], [0, 0, 9, 0, 0], [6, 0, 0, 0, 0], [0, 0, 0, 0, 0], [0, 0, 0, 0, 0]]),
+])
+def test_sparse_conv2d_hand_written_rectangles(padding, y_exp):
+    from sbnet_amd import sparse_conv as sc
+    ind_blk = torch.tensor(UPSAMPLE_EXP, dtype=torch.int32, device=DEV).view(2, 3, 3, 3)
+    x = torch.ones((1, 5, 5, 1), device=DEV)
+    w = torch.ones((3, 3, 1, 1), device=DEV)
+    y = sc.sparse_conv2d(x, w, ind_blk, [1, 1, 1, 1], padding)
+    y_exp = np.asarray(y_exp, np.float32)
+    assert y.numel() == y_exp.size
+    np.testing.assert_array_equal(y.cpu().numpy().reshape(y_exp.shape), y_exp)
+
+
+@pytest.mark.parametrize("case", GOLD["pipeline"], ids=lambda c: c["name"])
+def test_sparse_conv2d_with_mask_known_answers(case):
+    """SparseConv2DTests._test_sparse_conv2d_with_mask (sparse_conv_tests.py:195-321): mask -> block indices ->
+    sparse_conv2d of ones with a kernel of ones, all five tables, stride-2 and VALID ones included."""
+    from sbnet_amd import sparse_conv as sc
+    mask = torch.tensor(case["mask"], dtype=torch.float32, device=DEV)[None]
+    bsize, ksize = [1] + case["bsize"] + [1], case["ksize"] + [1, 1]
+    strides = [1] + case["conv_strides"] + [1]
+    ind_blk = sc.convert_mask_to_block_indices(mask, bsize, ksize, strides, case["padding"], 0.0)
+    assert ind_blk.dtype == torch.int32 and tuple(ind_blk.shape[1:]) == (case["bsize"][0], case["bsize"][1], 3)
+    x = torch.ones((1, mask.shape[1], mask.shape[2], 1), device=DEV)
+    w = torch.ones(tuple(ksize), device=DEV)
+    y = sc.sparse_conv2d(x, w, ind_blk, strides, case["padding"])
+    y_exp = np.asarray(case["y_exp"], np.float32)
+    assert y.numel() == y_exp.size
+    np.testing.assert_array_equal(y.cpu().numpy().reshape(y_exp.shape), y_exp)
+
+
+def _random_problem(kk, cout=10):
+    rng = np.random.RandomState(0)
+    xsize = [10, 28, 28, 10]
+    x = rng.uniform(-1, 1, xsize).astype(np.float32)
+    w = rng.uniform(-1, 1, [kk, kk, 10, cout]).astype(np.float32)
+    mask = (rng.uniform(-5, 1, xsize[:-1]) > 0).astype(np.float32)
+    return (torch.from_numpy(a).to(DEV) for a in (x, w, mask))
+
+
+def _compare_on_active_outputs(y_act, x, w, mask, strides, padding):
+    """The reference compares where the max-pooled mask is set (sparse_conv_tests.py:336-349) with rtol 1e-2 /
+    atol 0.1; fp32 convolutions agree far better, and outside the active rectangles the sparse result is 0."""
+    from sbnet_amd import sparse_conv as sc
+    y_exp = sc.mask_conv2d(x, w, mask, strides, padding)
+    kh, kw = int(w.shape[0]), int(w.shape[1])
+    m = sc._pool_same_or_valid(mask[:, None], (kh, kw), (strides[1], strides[2]), padding)[:, 0] > 0
+    assert y_act.shape == y_exp.shape and int(m.sum()) > 0
+    torch.testing.assert_close(y_act[m], y_exp[m], rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("ss", [1, 2])
+@pytest.mark.parametrize("padding", ["SAME", "VALID"])
+@pytest.mark.parametrize("kk", [1, 3, 5])
+def test_sparse_conv2d_matches_dense_conv(kk, padding, ss):
+    """SparseConv2DTests.test_sparse_conv2d_correctness (sparse_conv_tests.py:324-359): x [10,28,28,10], kernel
+    k in {1,3,5}, blocks of k+2, both paddings, strides 1 and 2."""
+    from sbnet_amd import sparse_conv as sc
+    x, w, mask = _random_problem(kk)
+    strides = [1, ss, ss, 1]
+    if (kk + 2 - kk) % ss != 0:
+        with pytest.raises(AssertionError):   # `stride` must divide `bsize` - `ksize`
+            sc.convert_mask_to_block_indices(mask, [1, kk + 2, kk + 2, 1], [kk, kk, 10, 10], strides, padding, 0.0)
+        return
+    ind_blk = sc.convert_mask_to_block_indices(mask, [1, kk + 2, kk + 2, 1], [kk, kk, 10, 10], strides, padding, 0.0)
+    y = sc.sparse_conv2d(x, w, ind_blk, strides, padding)
+    _compare_on_active_outputs(y, x, w, mask, strides, padding)
+
+
+@pytest.mark.parametrize("padding", ["SAME", "VALID"])
+@pytest.mark.parametrize("kk", [1, 3, 5])
+def test_sparse_conv2d_matmul_matches_dense_conv(kk, padding):
+    """SparseConv2DTests.test_sparse_conv2d_matmul_correctness (sparse_conv_tests.py:361-397): blocks of the
+    kernel's size, one output pixel each."""
+    from sbnet_amd import sparse_conv as sc
+    x, w, mask = _random_problem(kk, cout=7)
+    strides = [1, 1, 1, 1]
+    ind_blk = sc.convert_mask_to_block_indices(mask, [1, kk, kk, 1], [kk, kk, 10, 7], strides, padding, 0.0)
+    y = sc.sparse_conv2d_matmul(x, w, ind_blk, strides, padding)
+    _compare_on_active_outputs(y, x, w, mask, strides, padding)
+    # on these rectangles the two index-list convolutions compute the same thing
+    y2 = sc.sparse_conv2d(x, w, ind_blk, strides, padding)
+    torch.testing.assert_close(y, y2, rtol=1e-4, atol=1e-4)
+    with pytest.raises(ValueError):
+        sc.sparse_conv2d_matmul(x, w, ind_blk, [1, 2, 2, 1], padding)
+
+
+def test_index_list_interface_corner_cases():
+    from sbnet_amd import sparse_conv as sc
+    x, w, mask = _random_problem(3)
+    bsize, ksize, strides = [1, 5, 5, 1], [3, 3, 10, 10], [1, 1, 1, 1]
+    # no active block: an empty list and a zero result of the convolution's shape
+    none = sc.convert_mask_to_block_indices(torch.zeros_like(mask), bsize, ksize, strides, "SAME", 0.0)
+    assert tuple(none.shape) == (0, 5, 5, 3)
+    y = sc.sparse_conv2d(x, w, none, strides, "SAME")
+    assert tuple(y.shape) == (10, 28, 28, 10) and float(y.abs().max()) == 0.0
+    # a negative tolerance: the zeros of the padding count, so every block is active (tf.nn.max_pool over tf.pad)
+    every = sc.convert_mask_to_indices(torch.zeros_like(mask), bsize, ksize, strides, "SAME", -0.5)
+    assert every.shape[0] == 10 * 10 * 10   # 28 + 2 padded to 32 -> (32 - 5) // 3 + 1 = 10 blocks per axis
+    # The block grid is the custom op's (same windows, same order) with one more row and column of blocks: the
+    # index-list path pads the far side from the padded extent (sparse_conv_lib.py:170-174: 30 -> 32 rows, 10
+    # blocks), calc_block_params from the unpadded one (:370-374: 31 rows, 9 blocks).
+    import sbnet_amd
+    bp = sbnet_amd.calc_block_params([10, 28, 28, 10], bsize, ksize, strides, "SAME")
+    assert list(bp.bcount) == [9, 9]
+    ind = sc.convert_mask_to_indices_custom(mask, bp, 0.0)
+    lst = sc.convert_mask_to_indices(mask, bsize, ksize, strides, "SAME", 0.0).cpu().numpy()
+    assert lst[:, 1].max() == 9 and lst[:, 2].max() == 9
+    common = lst[(lst[:, 1] < 9) & (lst[:, 2] < 9)]
+    np.testing.assert_array_equal(common,
+                                  ind.active_block_indices[:int(ind.bin_counts[0])].cpu().numpy().astype(np.int32))
+    lst = torch.from_numpy(lst).to(DEV)
+    # rectangles must be rectangles
+    bad = sc.upsample_indices(lst[:4], bsize, [1, 3, 3, 1]).clone()
+    bad[1, 2, 2, 1] += 1
+    with pytest.raises(ValueError):
+        sc.sparse_conv2d(x, w, bad, strides, "SAME")
+
+
+def test_sparse_conv2d_gradients_match_the_masked_dense_convolution():
+    """Loss restricted to the active outputs: d/dw and d/dx through gather -> conv -> scatter equal those of the
+    dense convolution (the gradients of the block ops are the reference's compositions, sparse_conv_lib.py:80-147)."""
+    from sbnet_amd import sparse_conv as sc
+    x, w, mask = _random_problem(3)
+    strides, padding = [1, 1, 1, 1], "SAME"
+    ind_blk = sc.convert_mask_to_block_indices(mask, [1, 5, 5, 1], [3, 3, 10, 10], strides, padding, 0.0)
+    g = torch.Generator(device=DEV).manual_seed(3)
+    probe = torch.randn((10, 28, 28, 10), generator=g, device=DEV)
+    xs, ws = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    y = sc.sparse_conv2d(xs, ws, ind_blk, strides, padding)
+    # outputs a rectangle writes: the interior left after a VALID 3x3 convolution of each 5x5 block
+    out_mask = torch.zeros((10, 28, 28), device=DEV)
+    o = ind_blk[:, 0, 0, :].long()
+    for dh in range(3):
+        for dw in range(3):
+            hh, ww = o[:, 1] + dh, o[:, 2] + dw
+            ok = (hh < 28) & (ww < 28)
+            out_mask[o[ok, 0], hh[ok], ww[ok]] = 1.0
+    (y * probe).sum().backward()
+    xd, wd = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    yd = sc._conv_same_or_valid(xd.permute(0, 3, 1, 2), sc._hwio_to_oihw(wd), (1, 1), padding).permute(0, 2, 3, 1)
+    (yd * probe * out_mask[..., None]).sum().backward()
+    torch.testing.assert_close(y.detach(), (yd * out_mask[..., None]).detach(), rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(ws.grad, wd.grad, rtol=1e-3, atol=1e-3)
+    torch.testing.assert_close(xs.grad, xd.grad, rtol=1e-4, atol=1e-4)
