@@ -112,8 +112,20 @@ def _workspace(device, nbytes):
     return ws
 
 
-def reduce_mask(mask, dynamic_bcount, dynamic_bsize, dynamic_bstride, dynamic_boffset, tol, avgpool=False,
-                sync=True):
+def _param(dynamic, attr, name):
+    """The ops take their block parameters as `dynamic_b*` inputs (reduce_mask.cc:100-110, sparse_gather.cc:48-57);
+    the reference's README.md:53-107 and sample.py:42-43 spell the same int pairs `bsize=`, `bstride=`, `boffset=`
+    (and pass the block count second).  Both spellings are accepted; exactly one must be given."""
+    if dynamic is not None and attr is not None:
+        raise TypeError("pass either dynamic_%s or %s, not both" % (name, name))
+    value = dynamic if dynamic is not None else attr
+    if value is None:
+        raise TypeError("missing block parameter %s (dynamic_%s)" % (name, name))
+    return value
+
+
+def reduce_mask(mask, dynamic_bcount=None, dynamic_bsize=None, dynamic_bstride=None, dynamic_boffset=None, tol=None,
+                avgpool=False, sync=True, bcount=None, bsize=None, bstride=None, boffset=None):
     """ReduceMask (reduce_mask.cc:100-221).
 
     mask: float32 GPU tensor [N,H,W,1] or [N,H,W].  Returns (active_block_indices, bin_counts):
@@ -122,6 +134,11 @@ def reduce_mask(mask, dynamic_bcount, dynamic_bsize, dynamic_bstride, dynamic_bo
     count is left on the device (bin_counts is then a GPU tensor) and the call does not wait.
     """
     lib = _lib.load()
+    dynamic_bcount, dynamic_bsize = _param(dynamic_bcount, bcount, "bcount"), _param(dynamic_bsize, bsize, "bsize")
+    dynamic_bstride = _param(dynamic_bstride, bstride, "bstride")
+    dynamic_boffset = _param(dynamic_boffset, boffset, "boffset")
+    if tol is None:
+        raise TypeError("reduce_mask: tol is required (the op attribute has no default, reduce_mask.cc:102)")
     mask = _dev_f32(mask, "mask")
     if mask.dim() not in (3, 4) or (mask.dim() == 4 and mask.shape[3] != 1):
         raise InvalidArgument("mask must be [N,H,W,1] (or [N,H,W]), got %s" % (tuple(mask.shape),))
@@ -170,11 +187,13 @@ def reduce_mask_functor(mask, bcount, bsize, bstride, boffset, tol, avgpool=Fals
     return idx, count
 
 
-def sparse_gather(x, bin_counts, active_block_indices, dynamic_bsize, dynamic_bstride, dynamic_boffset,
-                  transpose=False, out=None):
+def sparse_gather(x, bin_counts, active_block_indices, dynamic_bsize=None, dynamic_bstride=None, dynamic_boffset=None,
+                  transpose=False, out=None, bsize=None, bstride=None, boffset=None):
     """SparseGather (sparse_gather.cc:48-57, 160-218): x [N,H,W,C] -> [M,bsize[0],bsize[1],C], or
     [M,C,bsize[0],bsize[1]] with transpose=True, M = bin_counts[0]; out-of-image pixels read as 0.
     Differentiable with respect to x (sparse_conv_lib.py:80-107)."""
+    dynamic_bsize, dynamic_bstride = _param(dynamic_bsize, bsize, "bsize"), _param(dynamic_bstride, bstride, "bstride")
+    dynamic_boffset = _param(dynamic_boffset, boffset, "boffset")
     if torch.is_grad_enabled() and isinstance(x, torch.Tensor) and x.requires_grad:
         if out is not None:
             raise ValueError("out= cannot be combined with a differentiable input")
@@ -277,11 +296,16 @@ def scatter_forward(x, bin_counts, active_block_indices, ybase, dynamic_bsize, d
         return y
 
 
-def sparse_scatter(x, bin_counts, active_block_indices, ybase, dynamic_bsize, dynamic_bstride, dynamic_boffset,
-                   add, atomic=False, transpose=False):
+def sparse_scatter(x, bin_counts, active_block_indices, ybase, dynamic_bsize=None, dynamic_bstride=None,
+                   dynamic_boffset=None, add=None, atomic=False, transpose=False, bsize=None, bstride=None,
+                   boffset=None):
     """SparseScatter (sparse_gather.cc:256-268, 286-357): returns copy(ybase) with the blocks of x written
     (add=False), added (add=True) or atomically added (add=True, atomic=True) on top.
     Differentiable with respect to x and ybase (sparse_conv_lib.py:110-147)."""
+    dynamic_bsize, dynamic_bstride = _param(dynamic_bsize, bsize, "bsize"), _param(dynamic_bstride, bstride, "bstride")
+    dynamic_boffset = _param(dynamic_boffset, boffset, "boffset")
+    if add is None:
+        raise TypeError("sparse_scatter: add is required (the op attribute has no default, sparse_gather.cc:258)")
     if torch.is_grad_enabled() and ((isinstance(x, torch.Tensor) and x.requires_grad) or
                                     (isinstance(ybase, torch.Tensor) and ybase.requires_grad)):
         from .autograd import SparseScatterFunction
@@ -292,10 +316,15 @@ def sparse_scatter(x, bin_counts, active_block_indices, ybase, dynamic_bsize, dy
                            dynamic_boffset, add, atomic, transpose, use_var=False)
 
 
-def sparse_scatter_var(x, bin_counts, active_block_indices, ybase, dynamic_bsize, dynamic_bstride,
-                       dynamic_boffset, add, atomic=False, transpose=False):
+def sparse_scatter_var(x, bin_counts, active_block_indices, ybase, dynamic_bsize=None, dynamic_bstride=None,
+                       dynamic_boffset=None, add=None, atomic=False, transpose=False, bsize=None, bstride=None,
+                       boffset=None):
     """SparseScatterVar (sparse_gather.cc:242-254, 335-337): the same, in place on ybase, which is returned.
     The reference registers no gradient for this op (its ybase is a variable reference); neither does this."""
+    dynamic_bsize, dynamic_bstride = _param(dynamic_bsize, bsize, "bsize"), _param(dynamic_bstride, bstride, "bstride")
+    dynamic_boffset = _param(dynamic_boffset, boffset, "boffset")
+    if add is None:
+        raise TypeError("sparse_scatter_var: add is required (the op attribute has no default, sparse_gather.cc:244)")
     if torch.is_grad_enabled() and ((isinstance(x, torch.Tensor) and x.requires_grad) or
                                     (isinstance(ybase, torch.Tensor) and ybase.requires_grad)):
         raise NotImplementedError("sparse_scatter_var has no gradient (none is registered for SparseScatterVar "

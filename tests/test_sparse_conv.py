@@ -402,3 +402,35 @@ def test_sparse_conv2d_gradients_match_the_masked_dense_convolution():
     torch.testing.assert_close(y.detach(), (yd * out_mask[..., None]).detach(), rtol=1e-4, atol=1e-4)
     torch.testing.assert_close(ws.grad, wd.grad, rtol=1e-3, atol=1e-3)
     torch.testing.assert_close(xs.grad, xd.grad, rtol=1e-4, atol=1e-4)
+
+
+def test_readme_attribute_spelling_and_sample():
+    """The reference's README.md:53-107 and sample.py:42-43 pass the block parameters as `bsize=`, `bstride=`,
+    `boffset=` (and the block count second); the op wrappers take both spellings, and the sample layer written that
+    way reproduces the dense convolution on the blocks it writes."""
+    import sbnet_amd
+    from sbnet_amd import sample
+    rng = np.random.default_rng(4)
+    mask = torch.from_numpy((rng.random((2, 20, 20, 1)) < 0.2).astype(np.float32)).to(DEV)
+    x = torch.from_numpy(rng.standard_normal((2, 20, 20, 8)).astype(np.float32)).to(DEV)
+    a = sbnet_amd.reduce_mask(mask, [5, 5], [6, 6], [4, 4], [-1, -1], 0.5)
+    b = sbnet_amd.reduce_mask(mask, [5, 5], bsize=[6, 6], boffset=[-1, -1], bstride=[4, 4], tol=0.5)
+    assert int(a.bin_counts[0]) == int(b.bin_counts[0]) > 0
+    assert torch.equal(a.active_block_indices[:int(a.bin_counts[0])], b.active_block_indices[:int(b.bin_counts[0])])
+    kw = dict(bsize=[6, 6], boffset=[-1, -1], bstride=[4, 4])
+    g1 = sbnet_amd.sparse_gather(x, a.bin_counts, a.active_block_indices, [6, 6], [4, 4], [-1, -1], transpose=True)
+    g2 = sbnet_amd.sparse_gather(x, a.bin_counts, a.active_block_indices, transpose=True, **kw)
+    assert torch.equal(g1, g2)
+    y1 = sbnet_amd.sparse_scatter(g1, a.bin_counts, a.active_block_indices, x, [6, 6], [4, 4], [-1, -1], add=True,
+                                  atomic=True, transpose=True)
+    y2 = sbnet_amd.sparse_scatter(g1, a.bin_counts, a.active_block_indices, x, add=True, atomic=True, transpose=True,
+                                  **kw)
+    assert torch.equal(y1, y2)
+    with pytest.raises(TypeError):
+        sbnet_amd.sparse_gather(x, a.bin_counts, a.active_block_indices, [6, 6], [4, 4], [-1, -1], bsize=[6, 6])
+    with pytest.raises(TypeError):
+        sbnet_amd.sparse_gather(x, a.bin_counts, a.active_block_indices, bsize=[6, 6], bstride=[4, 4])
+    with pytest.raises(TypeError):
+        sbnet_amd.sparse_scatter(g1, a.bin_counts, a.active_block_indices, x, **kw)   # add has no default
+    y = sample.main(seed=1, device=DEV)
+    assert tuple(y.shape) == (4, 254, 254, 64)
