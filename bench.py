@@ -290,7 +290,12 @@ def cxx_pipeline(path, steps, warmup, batches):
     so = os.path.join(ROOT, "sbnet_amd", "libsbnet_bench.so")
     if not os.path.exists(so):
         raise RuntimeError("%s is not built; run `make -C sbnet_amd/csrc`" % so)
-    loop = ctypes.CDLL(so).sbnet_bench_pipeline
+    lib_so = ctypes.CDLL(so)
+    lib_so.sbnet_bench_struct_bytes.restype = ctypes.c_size_t
+    if (lib_so.sbnet_bench_struct_bytes(0), lib_so.sbnet_bench_struct_bytes(1)) != \
+            (ctypes.sizeof(BenchSet), ctypes.sizeof(BenchGeom)):
+        raise RuntimeError("BenchSet / BenchGeom do not match the structs of sbnet_bench_loop.cpp; rebuild %s" % so)
+    loop = lib_so.sbnet_bench_pipeline
     loop.restype = ctypes.c_int
     loop.argtypes = [ctypes.POINTER(BenchSet), ctypes.c_int, ctypes.POINTER(BenchGeom), ctypes.c_int, ctypes.c_int,
                      ctypes.c_void_p, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int32)]

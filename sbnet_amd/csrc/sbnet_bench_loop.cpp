@@ -31,6 +31,13 @@ struct sbnet_bench_geom {
     int32_t max_active;
 };
 
+// sizeof of the two structs above (0: set, 1: geometry), for a caller that mirrors them in another language to
+// check its layout before passing pointers.
+size_t sbnet_bench_struct_bytes(int which)
+{
+    return which == 0 ? sizeof(sbnet_bench_set) : which == 1 ? sizeof(sbnet_bench_geom) : 0;
+}
+
 // Runs `steps` steps on `stream`, rotating over the sets, between two stream synchronisations; writes the elapsed
 // wall time in seconds and the count of the last step.  mode 0: the reference's contract (reduce_mask returns
 // with the count on the host, which sizes gather and scatter); mode 1: the count stays on the device.

@@ -54,3 +54,13 @@ def test_counters_of_another_kernel_source_are_not_reported(tmp_path, monkeypatc
     (prof / SUMMARY).write_text("\n".join(lines) + "\n")  # no digest at all: nothing to trust
     assert bench.read_measured_traffic(SUMMARY, "gather")[0] is None
     assert bench.read_measured_traffic("no_such_file.txt", "gather")[0] is None
+
+
+def test_bench_structs_match_the_cxx_loop():
+    """bench.py hands the C++ host loop two structs by pointer; their ctypes mirrors must have the C layout."""
+    import ctypes
+    so = os.path.join(ROOT, "sbnet_amd", "libsbnet_bench.so")
+    lib = ctypes.CDLL(so)
+    lib.sbnet_bench_struct_bytes.restype = ctypes.c_size_t
+    assert lib.sbnet_bench_struct_bytes(0) == ctypes.sizeof(bench.BenchSet) == 64
+    assert lib.sbnet_bench_struct_bytes(1) == ctypes.sizeof(bench.BenchGeom)

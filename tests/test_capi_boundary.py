@@ -28,6 +28,56 @@ def test_header_declares_what_the_loader_binds():
     assert declared_symbols() == sorted(_lib.SIGNATURES)
 
 
+def _c_kind(ctype):
+    """Coarse kind of a C parameter or return type as written in the header."""
+    t = " ".join(ctype.replace("const", " ").split())
+    if "*" in t:
+        return "char*" if t.startswith("char") else "ptr"
+    return {"int": "i32", "int32_t": "i32", "unsigned int": "u32", "uint32_t": "u32", "int64_t": "i64",
+            "size_t": "size", "float": "f32", "void": "void"}[t]
+
+
+def _ctypes_kind(t):
+    if t is None:
+        return "void"
+    if t is ctypes.c_char_p:
+        return "char*"
+    if t is ctypes.c_void_p or isinstance(t, type(ctypes.POINTER(ctypes.c_int))):
+        return "ptr"
+    return {ctypes.c_int: "i32", ctypes.c_int32: "i32", ctypes.c_uint: "u32", ctypes.c_uint32: "u32",
+            ctypes.c_int64: "i64", ctypes.c_size_t: "size", ctypes.c_float: "f32"}[t]
+
+
+def declared_signatures():
+    """name -> (kind of the return type, kinds of the parameters), parsed from the header's declarations."""
+    text = open(os.path.join(ROOT, "include", "sbnet_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"//[^\n]*", "", text)
+    out = {}
+    for ret, name, params in re.findall(r"([A-Za-z_][\w\s\*]*?)\b(sbnet_[a-z_]+)\s*\(([^)]*)\)\s*;", text):
+        kinds = []
+        for prm in params.split(","):
+            prm = " ".join(prm.split())
+            if prm in ("void", ""):
+                continue
+            m = re.match(r"(.*?)(\w+)$", prm)   # type, then the parameter's name
+            kinds.append(_c_kind(m.group(1)))
+        out[name] = (_c_kind(ret), kinds)
+    return out
+
+
+def test_loader_signatures_match_the_header_declarations():
+    """ctypes does not check a prototype: a parameter added on one side only would shift every argument after it.
+    Parameter count, order and width class (pointer / 32-bit / 64-bit / size_t / float) of every entry point, as
+    the header declares them, against what the loader binds."""
+    decl = declared_signatures()
+    assert sorted(decl) == sorted(_lib.SIGNATURES)
+    for name, (res, args) in _lib.SIGNATURES.items():
+        want_res, want_args = decl[name]
+        assert _ctypes_kind(res) == want_res, name
+        assert [_ctypes_kind(a) for a in args] == want_args, name
+
+
 def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(_lib.LIB_PATH)
     for name in declared_symbols():
