@@ -1,5 +1,5 @@
 // C ABI of libsbnet_amd.so (declared in include/sbnet_amd.h): argument validation that mirrors
-// the reference ops' OP_REQUIRES checks, then the kernel launches of sbnet_kernels.hip.
+// the reference ops' OP_REQUIRES checks, then the kernel launches of sbnet_reduce_mask.hip, sbnet_gather.hip and sbnet_scatter.hip.
 //
 // Reference behaviour reproduced here (sbnet_tensorflow/sbnet_ops/):
 //   reduce_mask.cc:132-138, 141-220   parameter shape check, host-visible count, zero-count fix-up

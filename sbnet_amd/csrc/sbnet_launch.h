@@ -1,5 +1,5 @@
 // Host-side launch interface between the C ABI (sbnet_capi.cpp) and the gfx950 kernels
-// (sbnet_kernels.hip).  Everything here takes already-validated arguments.
+// (sbnet_reduce_mask.hip, sbnet_gather.hip, sbnet_scatter.hip).  Everything here takes already-validated arguments.
 #pragma once
 
 #include <hip/hip_runtime_api.h>
@@ -45,7 +45,7 @@ hipError_t launch_reduce_mask(const float* mask, const Geom& g, int bCntH, int b
 constexpr size_t STATIC_SCRATCH_BYTES = (size_t)2 << 20;
 hipError_t static_scratch(void** ptr);
 
-// Test hook: see tile_choice in sbnet_kernels.hip.
+// Test hook: see tile_choice in sbnet_gather.hip.
 int tile_choice(int kind, const Geom& g, int numActive, int vec, int yAlignedTo, int32_t* out);
 
 hipError_t launch_gather(const float* x, float* y, const int16_t* idx, int numActive,

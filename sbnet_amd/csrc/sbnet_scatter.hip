@@ -1,0 +1,1087 @@
+// sparse_scatter / sparse_scatter_var on gfx950: plain write, add and atomic add from either stack layout; the
+// owner-computes overlapping add, the add in passes, ordered overlapping writes (rank table, owner map), the
+// copying op built in one pass, and the flat copy; with the launch configuration.
+// Reference semantics: sbnet_tensorflow/sbnet_ops/sparse_gather.cc:103-130, 135-142, 338-346.
+#include "sbnet_device.h"
+
+namespace sbnet {
+
+// sparse_gather.cc:103-130 with transpose == false.
+template <int VEC, int MODE>
+__global__ __launch_bounds__(256) void k_scatter_nhwc_wide(const float* __restrict__ x, float* y, const float* ysrc,
+                                                      const int16_t* __restrict__ idx, NhwcArgs a, ColorArgs col)
+{
+    typedef typename Vec<VEC>::type vec;
+    const uint32_t lane = threadIdx.x & 63;
+    uint32_t unit = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (unit >= a.units) return;
+    unit = __builtin_amdgcn_readfirstlane(unit);
+    const uint32_t ib = fdiv(unit, a.dCpb);
+    if (beyond_count(a.g, ib)) return;
+    const uint32_t chunk = unit - ib * a.cpb;
+    const BlockOrigin o = origin_of(load_triple(idx, ib), a.g);  // ib is wave-uniform: scalar load
+    if (!o.valid) return;
+    bool atomics = MODE == SCATTER_ATOMIC;
+    if (MODE == SCATTER_COLOR && color_skip(col, o, atomics)) return;
+    const int CV = a.g.C / VEC;
+    const int slo = max(0, -o.w0), shi = min(a.g.S, a.g.W - o.w0);
+    const int lo = slo * CV, hi = shi * CV;
+    const vec* __restrict__ xb = reinterpret_cast<const vec*>(x) + (size_t)ib * a.blockV;
+    vec* yv = reinterpret_cast<vec*>(y);
+    const vec* ysv = reinterpret_cast<const vec*>(ysrc);  // what an add reads: y itself, or the base y is a copy of
+    const uint32_t e0 = chunk * NHWC_CHUNK + lane;
+
+    vec v[NHWC_UNR];
+    int64_t dst[NHWC_UNR];
+#pragma unroll
+    for (int u = 0; u < NHWC_UNR; ++u) {
+        const uint32_t e = e0 + u * 64;
+        dst[u] = -1;
+        v[u] = vzero<VEC>();
+        if (e < a.blockV) {
+            const uint32_t r = fdiv(e, a.dRow);
+            const int j = (int)(e - r * a.rowV);
+            const int hh = o.h0 + (int)r;
+            if ((unsigned)hh < (unsigned)a.g.H && j >= lo && j < hi) {
+                dst[u] = (((int64_t)o.n * a.g.H + hh) * a.g.W + o.w0) * CV + j;
+                if (MODE == SCATTER_OWNED &&
+                    col.owner[((int64_t)o.n * a.g.H + hh) * a.g.W + o.w0 + (int)fdiv((uint32_t)j, a.dCV)] != (int32_t)ib)
+                    dst[u] = -1;
+                else if (MODE == SCATTER_RANKED && ranked_out(rank_bits(col, ib), r, fdiv((uint32_t)j, a.dCV), a.g))
+                    dst[u] = -1;
+                else
+                    v[u] = ld_stream(xb + e);
+            }
+        }
+    }
+    if (MODE == SCATTER_ADD || (MODE == SCATTER_COLOR && !atomics)) {
+        vec cur[NHWC_UNR];
+#pragma unroll
+        for (int u = 0; u < NHWC_UNR; ++u)
+            if (dst[u] >= 0) cur[u] = ld_stream(ysv + dst[u]);
+#pragma unroll
+        for (int u = 0; u < NHWC_UNR; ++u)
+            if (dst[u] >= 0) st_stream(yv + dst[u], vadd(cur[u], v[u]));
+    } else if (MODE == SCATTER_ASSIGN || MODE == SCATTER_OWNED || MODE == SCATTER_RANKED) {
+#pragma unroll
+        for (int u = 0; u < NHWC_UNR; ++u)
+            if (dst[u] >= 0) commit<VEC, SCATTER_ASSIGN>(yv + dst[u], v[u]);
+    } else {
+#pragma unroll
+        for (int u = 0; u < NHWC_UNR; ++u)
+            if (dst[u] >= 0) commit<VEC, SCATTER_ATOMIC>(yv + dst[u], v[u]);
+    }
+}
+
+template <int VEC, int MODE>
+__global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ x, float* y, const float* ysrc,
+                                                      const int16_t* __restrict__ idx, NhwcArgs a, ColorArgs col)
+{
+    typedef typename Vec<VEC>::type vec;
+    const uint32_t lane = threadIdx.x & 63;
+    uint32_t unit = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (unit >= a.units) return;
+    unit = __builtin_amdgcn_readfirstlane(unit);
+    const uint32_t ib = fdiv(unit, a.dCpb);
+    if (beyond_count(a.g, ib)) return;
+    const uint32_t chunk = unit - ib * a.cpb;
+    const BlockOrigin o = origin_of(load_triple(idx, ib), a.g);
+    if (!o.valid) return;
+    bool atomics = MODE == SCATTER_ATOMIC;
+    if (MODE == SCATTER_COLOR && color_skip(col, o, atomics)) return;
+    const int CV = a.g.C / VEC;
+    const int slo = max(0, -o.w0), shi = min(a.g.S, a.g.W - o.w0);
+    const int lo = slo * CV, hi = shi * CV;
+    const int64_t imgFloats = (int64_t)a.g.H * a.g.W * a.g.C;
+    float* img = y + (int64_t)o.n * imgFloats;
+    const rsrc_t yr = make_rsrc(img, (uint32_t)imgFloats * 4u);
+    const rsrc_t sr = make_rsrc(ysrc + (int64_t)o.n * imgFloats, (uint32_t)imgFloats * 4u);  // what an add reads
+    const rsrc_t xr = make_rsrc(x + (int64_t)ib * a.blockV * VEC, a.blockV * (uint32_t)(VEC * 4));
+    const uint32_t e0 = chunk * NHWC_CHUNK + lane;
+    vec v[NHWC_UNR];
+    uint32_t dst[NHWC_UNR];
+    int32_t own[NHWC_UNR];
+    const rsrc_t wr = make_rsrc(MODE == SCATTER_OWNED ? col.owner + (int64_t)o.n * a.g.H * a.g.W : nullptr,
+                                MODE == SCATTER_OWNED ? (uint32_t)(a.g.H * a.g.W) * 4u : 0u);
+#pragma unroll
+    for (int u = 0; u < NHWC_UNR; ++u) {
+        const uint32_t e = e0 + u * 64;
+        const uint32_t r = fdiv(e, a.dRow);
+        const int j = (int)(e - r * a.rowV);
+        const int hh = o.h0 + (int)r;
+        bool ok = e < a.blockV && (unsigned)hh < (unsigned)a.g.H && j >= lo && j < hi;
+        if (MODE == SCATTER_RANKED) ok = ok && !ranked_out(rank_bits(col, ib), r, fdiv((uint32_t)j, a.dCV), a.g);
+        dst[u] = ok ? (((uint32_t)hh * (uint32_t)a.g.W + (uint32_t)o.w0) * (uint32_t)CV + (uint32_t)j) * (uint32_t)(VEC * 4)
+                    : BUF_OOB;
+        v[u] = buf_load<VEC>(xr, ok ? e * (uint32_t)(VEC * 4) : BUF_OOB);  // off-image parts are not read
+        if (MODE == SCATTER_OWNED) {
+            const uint32_t pix = (uint32_t)hh * (uint32_t)a.g.W + (uint32_t)o.w0 + fdiv((uint32_t)j, a.dCV);
+            own[u] = __builtin_bit_cast(int32_t, buf_load<1>(wr, ok ? pix * 4u : BUF_OOB));
+        }
+    }
+    if (MODE == SCATTER_OWNED) {
+        // (an out-of-range owner read returns 0, which may equal ib: dst is BUF_OOB there already)
+#pragma unroll
+        for (int u = 0; u < NHWC_UNR; ++u) buf_store<BUF_NT>(yr, own[u] == (int32_t)ib ? dst[u] : BUF_OOB, v[u]);
+    } else if (MODE == SCATTER_ASSIGN || MODE == SCATTER_RANKED) {
+#pragma unroll
+        for (int u = 0; u < NHWC_UNR; ++u) buf_store<BUF_NT>(yr, dst[u], v[u]);
+    } else if (MODE == SCATTER_ADD || (MODE == SCATTER_COLOR && !atomics)) {
+        vec cur[NHWC_UNR];
+#pragma unroll
+        for (int u = 0; u < NHWC_UNR; ++u) cur[u] = buf_load<VEC>(sr, dst[u]);
+#pragma unroll
+        for (int u = 0; u < NHWC_UNR; ++u) buf_store<BUF_NT>(yr, dst[u], vadd(cur[u], v[u]));
+    } else {
+#pragma unroll
+        for (int u = 0; u < NHWC_UNR; ++u) {
+            if (dst[u] != BUF_OOB) {
+                float* d = img + (dst[u] >> 2);
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) atomic_add_f32(d + k, vget(v[u], k));
+            }
+        }
+    }
+}
+
+// sparse_gather.cc:103-130 with transpose == true: the block stack is [blocks, C, R, S].
+template <int VEC, int MODE, typename G>
+__device__ __forceinline__ void scatter_planar_tile(const float* __restrict__ x, float* y, const float* ysrc,
+                                                    const int16_t* __restrict__ idx, const TileArgs& a,
+                                                    const ColorArgs& col, float* lds, uint32_t ib, uint32_t rem)
+{
+    typedef typename Vec<VEC>::type vec;
+    const uint32_t tid = threadIdx.x, nthr = G::nthr(a);
+    const uint32_t RS = G::RS(a), Pp = G::Pp(a), vpr = G::vpr(a);
+    TileId t;
+    decode_tile<G>(a, t, ib, rem);
+    const RawTriple raw = load_triple(idx, t.ib);  // scalar load, needed only after the barrier
+    if (beyond_count(a.g, t.ib)) return;
+    bool atomics = MODE == SCATTER_ATOMIC;
+    if (MODE == SCATTER_COLOR && color_skip(col, origin_of(raw, a.g), atomics)) return;  // (here: before the loads)
+
+    // global -> registers, planar side.  The last slot of a run, when partial, is read as the last 4 floats
+    // of the run instead (overlapping its neighbour): no load leaves the run, no value needs fixing up.
+    const rsrc_t xr = make_rsrc(x + ((int64_t)t.ib * G::C(a) + t.c0) * RS + t.p0,
+                                ((uint32_t)(t.ctEff - 1) * RS + (uint32_t)t.Pn) * 4u);
+    const uint32_t slots = (uint32_t)t.ctEff * vpr;
+    if (t.Pn >= 4) {
+        f4 val[TILE_LD];
+#pragma unroll
+        for (int u = 0; u < TILE_LD; ++u) {
+            const uint32_t i = u * nthr + tid;
+            const uint32_t c = G::divVpr(i, a);
+            const int e0 = min(4 * (int)(i - c * vpr), t.Pn - 4);
+            val[u] = buf_load<4>(xr, i < slots ? (c * RS + (uint32_t)e0) * 4u : BUF_OOB);
+        }
+#pragma unroll
+        for (int u = 0; u < TILE_LD; ++u) {
+            const uint32_t i = u * nthr + tid;
+            if (i < slots) {
+                const uint32_t c = G::divVpr(i, a);
+                const int e0 = 4 * (int)(i - c * vpr);
+                float* __restrict__ row = lds + c * Pp;
+                if (e0 + 4 <= t.Pn) {
+                    *reinterpret_cast<f4*>(row + ((uint32_t)e0 ^ lds_swz(c))) = val[u];
+                } else if (e0 < t.Pn) {  // partial last slot: holds floats [Pn-4, Pn) of the run
+                    const uint32_t t0 = (uint32_t)(t.Pn - 4);
+                    row[(t0 + 0) ^ lds_swz(c)] = val[u].x;
+                    row[(t0 + 1) ^ lds_swz(c)] = val[u].y;
+                    row[(t0 + 2) ^ lds_swz(c)] = val[u].z;
+                    row[(t0 + 3) ^ lds_swz(c)] = val[u].w;
+                }
+            }
+        }
+    } else {
+        // A plane's last split can hold fewer pixels than one slot (the split width is rounded up to whole slots,
+        // and 1-3 pixels may remain): one thread per row moves them float by float.
+        if (tid < (uint32_t)t.ctEff) {
+            for (int k = 0; k < t.Pn; ++k)
+                lds[tid * Pp + ((uint32_t)k ^ lds_swz(tid))] = buf_load<1>(xr, (tid * RS + (uint32_t)k) * 4u);
+        }
+    }
+    lds_barrier();
+
+    // NHWC side: LDS -> base tensor; pixels outside the image are dropped (sparse_gather.cc:121)
+    const BlockOrigin o = origin_of(raw, a.g);
+    if (!o.valid) return;
+    float* img = y + (int64_t)o.n * a.imgFloats;
+    const rsrc_t yr = make_rsrc(img, a.imgBytes);
+    const rsrc_t sr = make_rsrc(ysrc + (int64_t)o.n * a.imgFloats, a.imgBytes);  // what an add reads
+    const uint32_t c0l = (tid & ((1u << G::lppLog(a)) - 1u)) * VEC;
+    vec w[TILE_LD];
+    uint32_t offs[TILE_LD];
+    int32_t own[TILE_LD];
+    const rsrc_t wr = make_rsrc(MODE == SCATTER_OWNED ? col.owner + (int64_t)o.n * a.g.H * a.g.W : nullptr,
+                                MODE == SCATTER_OWNED ? (uint32_t)(a.g.H * a.g.W) * 4u : 0u);
+    const uint32_t rbits = MODE == SCATTER_RANKED ? rank_bits(col, t.ib) : 0u;
+    nhwc_walk<VEC, G>(a, t, o, tid, nthr, [&](int u, uint32_t pl, uint32_t off, uint32_t pix, uint32_t r, uint32_t sc) {
+        if (MODE == SCATTER_RANKED && ranked_out(rbits, r, sc, a.g)) off = BUF_OOB;
+        offs[u] = off;
+        if (MODE == SCATTER_OWNED) own[u] = __builtin_bit_cast(int32_t, buf_load<1>(wr, off != BUF_OOB ? pix * 4u : BUF_OOB));
+        w[u] = vzero<VEC>();
+        if (off != BUF_OOB) {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                const uint32_t c = c0l + k;
+                vset(w[u], k, lds[c * Pp + (pl ^ lds_swz(c))]);
+            }
+        }
+    });
+    if (MODE == SCATTER_OWNED) {
+#pragma unroll
+        for (int u = 0; u < TILE_LD; ++u) buf_store<BUF_NT>(yr, own[u] == (int32_t)t.ib ? offs[u] : BUF_OOB, w[u]);
+    } else if (MODE == SCATTER_ASSIGN || MODE == SCATTER_RANKED) {
+#pragma unroll
+        for (int u = 0; u < TILE_LD; ++u) buf_store<BUF_NT>(yr, offs[u], w[u]);
+    } else if (MODE == SCATTER_ADD || (MODE == SCATTER_COLOR && !atomics)) {
+        vec cur[TILE_LD];
+#pragma unroll
+        for (int u = 0; u < TILE_LD; ++u) cur[u] = buf_load<VEC>(sr, offs[u]);
+#pragma unroll
+        for (int u = 0; u < TILE_LD; ++u) buf_store<BUF_NT>(yr, offs[u], vadd(cur[u], w[u]));
+    } else {
+#pragma unroll
+        for (int u = 0; u < TILE_LD; ++u) {
+            if (offs[u] != BUF_OOB) {
+                float* d = img + (offs[u] >> 2);
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) atomic_add_f32(d + k, vget(w[u], k));
+            }
+        }
+    }
+}
+
+template <int VEC, int MODE, typename G>
+__global__ __launch_bounds__(512) void k_scatter_planar(const float* __restrict__ x, float* y, const float* ysrc,
+                                                        const int16_t* __restrict__ idx, TileArgs a, ColorArgs col)
+{
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    for_each_block_of_workgroup(a, G::tpb(a), [&](uint32_t ib, uint32_t rem) {
+        scatter_planar_tile<VEC, MODE, G>(x, y, ysrc, idx, a, col, lds, ib, rem);
+    });
+}
+
+// ---------------------------------------------------------------------------------------------
+// overlapping scatter-add without atomics: every output pixel is summed by one owner
+// ---------------------------------------------------------------------------------------------
+//
+// With bstride < bsize a pixel is covered by up to ceil(R/U)*ceil(S/V) blocks.  Hardware fp32 atomics
+// resolve that at roughly a tenth of the HBM rate (every contribution is a read-modify-write in L2) and
+// in arbitrary order.  Given a little scratch memory the add is done by "pulling" instead:
+//   1. k_pull_fill / k_pull_map   an inverse map (n, bh, bw) -> position ib in the active list;
+//   2. k_pull_table               per active block, the active blocks that overlap it, sorted by ib;
+//   3. k_scatter_pull             the workgroup of block ib walks its own pixels; a pixel belongs to the
+//                                 lowest-ib block that covers it, and that owner reads the pixel once,
+//                                 adds the contributions of all covering blocks in ascending ib order
+//                                 and writes it once.
+// Ascending ib is the order in which the sequential CPU functor accumulates (sparse_gather.cc:105-129),
+// so the result is bit-identical to it and reproducible from run to run.  A block listed twice cannot
+// be represented in the map; k_pull_map notices, and k_scatter_pull then falls back to hardware atomics
+// for the whole launch (still correct, to rounding).
+
+constexpr int PULL_STEPS = 3;    // 64-vector steps of one wave, all in flight together (1: 223 us, 2: 228, 3: 211, 4: 232
+                                 // on the 16x16-at-stride-8, 256-channel workload; 5 and more run out of registers)
+constexpr int PULL_CLASSES = 9;  // 3 row classes x 3 column classes of a block's pixels (see below)
+constexpr int PULL_COVER = 4;    // at most 2 x 2 blocks cover a pixel
+constexpr int PULL_TABLE_STRIDE = PULL_CLASSES * PULL_COVER * 2;  // ints per block
+
+// With at most 2x2 blocks over a pixel, which blocks cover a pixel of block (bh, bw) depends only on the pixel's
+// class: its row is among the first R-U rows (shared with the blocks one step up), among the rows from U on (one
+// step down) or in between (this row of blocks only), and the same for columns.  The table holds, per block and
+// class, the up to four active blocks that cover pixels of the class, sorted by list position, each as (position,
+// packed grid offset): the main kernel needs no search, and the first entry names the pixel's owner.
+
+struct PullArgs {
+    Geom g;
+    int bhMin, bwMin, nBH, nBW;  // extent of the inverse map: blocks that can touch the image
+    int kh1, kw1;                // Kh - 1, Kw - 1
+    uint32_t CV, rowV, blockV;   // vectors per pixel, per block row, per block
+    uint32_t cpb, units;         // wave-units per block, in total
+    FastDiv dCpb, dRow, dCV;
+};
+
+__global__ __launch_bounds__(256) void k_pull_fill(int32_t* __restrict__ map, int64_t n, int32_t* __restrict__ dup)
+{
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) map[i] = -1;
+    if (blockIdx.x == 0 && threadIdx.x == 0) *dup = 0;
+}
+
+__device__ __forceinline__ int64_t pull_slot(const PullArgs& a, int n, int bh, int bw)
+{
+    if ((unsigned)n >= (unsigned)a.g.N) return -1;
+    const int ih = bh - a.bhMin, iw = bw - a.bwMin;
+    if ((unsigned)ih >= (unsigned)a.nBH || (unsigned)iw >= (unsigned)a.nBW) return -1;
+    return ((int64_t)n * a.nBH + ih) * a.nBW + iw;
+}
+
+__global__ __launch_bounds__(256) void k_pull_map(const int16_t* __restrict__ idx, int numActive, PullArgs a,
+                                                  int32_t* __restrict__ map, int32_t* __restrict__ dup)
+{
+    const int ib = (int)(blockIdx.x * 256 + threadIdx.x);
+    if (ib >= numActive || (a.g.countDev && ib >= *a.g.countDev)) return;
+    const int64_t slot = pull_slot(a, idx[(size_t)ib * 3], idx[(size_t)ib * 3 + 1], idx[(size_t)ib * 3 + 2]);
+    if (slot < 0) return;  // this block cannot touch the image
+    if (atomicCAS(map + slot, -1, ib) != -1) *dup = 1;
+}
+
+// One thread per (block, class): the up to four active blocks that cover the class's pixels, sorted by position.
+__global__ __launch_bounds__(256) void k_pull_table(const int16_t* __restrict__ idx, int numActive, PullArgs a,
+                                                    const int32_t* __restrict__ map, int32_t* __restrict__ table)
+{
+    const uint32_t t = blockIdx.x * 256u + threadIdx.x;
+    const int ib = (int)(t / PULL_CLASSES), cls = (int)(t % PULL_CLASSES);
+    if (ib >= numActive || (a.g.countDev && ib >= *a.g.countDev)) return;
+    const int n = idx[(size_t)ib * 3], bh = idx[(size_t)ib * 3 + 1], bw = idx[(size_t)ib * 3 + 2];
+    const int rc = cls / 3, cc = cls - rc * 3;
+    // a block one step up covers the first R-U rows only (row class 0), one step down the rows from U on (class 2)
+    const int dhLo = rc == 0 ? -a.kh1 : 0, dhHi = rc == 2 ? a.kh1 : 0;
+    const int dwLo = cc == 0 ? -a.kw1 : 0, dwHi = cc == 2 ? a.kw1 : 0;
+    int ids[PULL_COVER], pks[PULL_COVER];
+    int cnt = 0;
+    if (pull_slot(a, n, bh, bw) >= 0) {
+        for (int dh = dhLo; dh <= dhHi; ++dh)
+            for (int dw = dwLo; dw <= dwHi; ++dw) {
+                const int64_t slot = pull_slot(a, n, bh + dh, bw + dw);
+                const int other = slot >= 0 ? map[slot] : -1;
+                if (other < 0) continue;
+                int k = cnt++;  // insertion sort
+                while (k > 0 && ids[k - 1] > other) {
+                    ids[k] = ids[k - 1];
+                    pks[k] = pks[k - 1];
+                    --k;
+                }
+                ids[k] = other;
+                pks[k] = ((dh & 0xffff) << 16) | (dw & 0xffff);
+            }
+    }
+    typedef int i4 __attribute__((ext_vector_type(4)));
+    int e[PULL_COVER * 2];
+#pragma unroll
+    for (int k = 0; k < PULL_COVER; ++k) {
+        e[2 * k] = k < cnt ? ids[k] : -1;
+        e[2 * k + 1] = k < cnt ? pks[k] : 0;
+    }
+    i4* q = reinterpret_cast<i4*>(table + (size_t)ib * PULL_TABLE_STRIDE + cls * (PULL_COVER * 2));
+    q[0] = (i4){e[0], e[1], e[2], e[3]};
+    q[1] = (i4){e[4], e[5], e[6], e[7]};
+}
+
+// sparse_gather.cc:103-130 with add == true on overlapping blocks, NHWC stack.
+template <int VEC>
+__global__ __launch_bounds__(256) void k_scatter_pull(const float* __restrict__ x, float* __restrict__ y,
+                                                      const int16_t* __restrict__ idx, PullArgs a,
+                                                      const int32_t* __restrict__ table,
+                                                      const int32_t* __restrict__ dup)
+{
+    typedef typename Vec<VEC>::type vec;
+    const uint32_t lane = threadIdx.x & 63;
+    uint32_t unit = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (unit >= a.units) return;
+    unit = __builtin_amdgcn_readfirstlane(unit);
+    const uint32_t ib = fdiv(unit, a.dCpb);
+    if (beyond_count(a.g, ib)) return;
+    const uint32_t chunk = unit - ib * a.cpb;
+    const BlockOrigin o = origin_of(load_triple(idx, ib), a.g);  // ib is wave-uniform: scalar load
+    if (!o.valid) return;
+    const vec* __restrict__ xv = reinterpret_cast<const vec*>(x);
+    vec* __restrict__ yv = reinterpret_cast<vec*>(y);
+
+    if (*dup != 0) {
+        // the list names a block twice: the map cannot represent it; hardware atomics for the whole launch
+        for (int step = 0; step < PULL_STEPS; ++step) {
+            const uint32_t e = (chunk * PULL_STEPS + step) * 64 + lane;
+            if (e >= a.blockV) break;
+            const uint32_t r = fdiv(e, a.dRow);
+            const uint32_t j = e - r * a.rowV;
+            const uint32_t s = fdiv(j, a.dCV);
+            const int hh = o.h0 + (int)r, ww = o.w0 + (int)s;
+            if ((unsigned)hh >= (unsigned)a.g.H || (unsigned)ww >= (unsigned)a.g.W) continue;
+            vec* dst = yv + ((((int64_t)o.n * a.g.H + hh) * a.g.W + ww) * a.CV + (j - s * a.CV));
+            commit<VEC, SCATTER_ATOMIC>(dst, ld_stream(xv + ((size_t)ib * a.blockV + e)));
+        }
+        return;
+    }
+
+    // Phase 1: per vector, its class's table entries (two 16-byte loads from a table line that the whole block shares).
+    const int32_t* __restrict__ t = table + (size_t)ib * PULL_TABLE_STRIDE;
+    typedef int i4 __attribute__((ext_vector_type(4)));
+    i4 ent[PULL_STEPS][2];
+    uint32_t rr[PULL_STEPS], ss[PULL_STEPS], cvv[PULL_STEPS];
+    bool in[PULL_STEPS];
+#pragma unroll
+    for (int u = 0; u < PULL_STEPS; ++u) {
+        const uint32_t e = (chunk * PULL_STEPS + u) * 64 + lane;
+        const uint32_t r = fdiv(e, a.dRow);
+        const uint32_t j = e - r * a.rowV;
+        const uint32_t s = fdiv(j, a.dCV);
+        rr[u] = r;
+        ss[u] = s;
+        cvv[u] = j - s * a.CV;
+        const int hh = o.h0 + (int)r, ww = o.w0 + (int)s;
+        in[u] = e < a.blockV && (unsigned)hh < (unsigned)a.g.H && (unsigned)ww < (unsigned)a.g.W;
+        const uint32_t rc = (int)r < a.g.R - a.g.U ? 0u : ((int)r >= a.g.U ? 2u : 1u);
+        const uint32_t cc = (int)s < a.g.S - a.g.V ? 0u : ((int)s >= a.g.V ? 2u : 1u);
+        const i4* q = reinterpret_cast<const i4*>(t + (in[u] ? (rc * 3u + cc) * (PULL_COVER * 2) : 0u));
+        ent[u][0] = q[0];
+        ent[u][1] = q[1];
+    }
+    // Phase 2: the owner of a pixel (the first of the blocks that cover it) reads the pixel and every contribution.
+    vec acc[PULL_STEPS], val[PULL_STEPS][PULL_COVER];
+    bool mine[PULL_STEPS], has[PULL_STEPS][PULL_COVER];
+    int64_t dstOff[PULL_STEPS];
+#pragma unroll
+    for (int u = 0; u < PULL_STEPS; ++u) {
+        const int id[PULL_COVER] = {ent[u][0].x, ent[u][0].z, ent[u][1].x, ent[u][1].z};
+        const int pk[PULL_COVER] = {ent[u][0].y, ent[u][0].w, ent[u][1].y, ent[u][1].w};
+        mine[u] = in[u] && id[0] == (int)ib;
+        const int hh = o.h0 + (int)rr[u], ww = o.w0 + (int)ss[u];
+        dstOff[u] = (((int64_t)o.n * a.g.H + hh) * a.g.W + ww) * a.CV + cvv[u];
+        // (loads under their own conditions: a load that no lane of the wave needs is skipped, and at one block
+        // in four active most pixels have one or two contributions, not four)
+        acc[u] = vzero<VEC>();
+        if (mine[u]) acc[u] = ld_stream(yv + dstOff[u]);
+#pragma unroll
+        for (int k = 0; k < PULL_COVER; ++k) {
+            has[u][k] = mine[u] && id[k] >= 0;
+            const int rs = (int)rr[u] - (int)(int16_t)(pk[k] >> 16) * a.g.U;
+            const int cs = (int)ss[u] - (int)(int16_t)(pk[k] & 0xffff) * a.g.V;
+            const int64_t off = (int64_t)id[k] * a.blockV + (int64_t)rs * a.rowV + (int64_t)cs * a.CV + cvv[u];
+            val[u][k] = vzero<VEC>();
+            if (has[u][k]) val[u][k] = ld_stream(xv + off);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < PULL_STEPS; ++u) {
+#pragma unroll
+        for (int k = 0; k < PULL_COVER; ++k)
+            if (has[u][k]) acc[u] = vadd(acc[u], val[u][k]);  // ascending list position: the CPU functor's order
+        if (mine[u]) st_stream(yv + dstOff[u], acc[u]);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// flat copy (CopyTensorFunctor, sparse_gather.cc:135-142 / sparse_gather.cu:268-276)
+// ---------------------------------------------------------------------------------------------
+
+constexpr int COPY_UNR = 4;  // 16 KB per workgroup; 32 KB per workgroup measured 30 % slower
+
+__global__ __launch_bounds__(256) void k_copy_v4(const f4* __restrict__ src, f4* __restrict__ dst, size_t n4)
+{
+    const size_t base = (size_t)blockIdx.x * (256 * COPY_UNR) + threadIdx.x;
+    f4 v[COPY_UNR];
+#pragma unroll
+    for (int u = 0; u < COPY_UNR; ++u) {
+        const size_t i = base + (size_t)u * 256;
+        v[u] = (f4)(0.f);
+        if (i < n4) v[u] = ld_stream(src + i);
+    }
+#pragma unroll
+    for (int u = 0; u < COPY_UNR; ++u) {
+        const size_t i = base + (size_t)u * 256;
+        if (i < n4) st_stream(dst + i, v[u]);
+    }
+}
+
+__global__ __launch_bounds__(256) void k_copy_scalar(const float* __restrict__ src, float* __restrict__ dst, size_t n)
+{
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) dst[i] = src[i];
+}
+
+// Tile of the planar scatter.  16 KB tiles suit a launch that keeps every compute unit busy for several
+// rounds of workgroups; a launch of few workgroups finishes in one or two rounds, where the loads and the stores
+// of one round do not overlap much, and does better with 24 KB tiles (800x800x128 tensor, 27x27 blocks:
+// 9.08 -> 8.87 us at 58 blocks, 20.6 -> 19.9 us at 156, but 40.8 -> 41.4 us at 312).
+constexpr int SCATTER_FEW_WGS_PER_CU = 22;
+
+// `share`: the launch does work for one block in `share` only (the passes of an overlapping add).
+static bool scatter_tile_args(const Geom& g, int numActive, int vec, TileArgs& a, int& threads, size_t& ldsBytes,
+                              unsigned& grid, int share = 1)
+{
+    if (!make_tile_args(g, numActive, vec, a, threads, ldsBytes, grid, 16 * 1024)) return false;
+    if (a.psplit > 1 && a.total / (uint32_t)share < (uint32_t)(SCATTER_FEW_WGS_PER_CU * device_cus())) {
+        TileArgs b;
+        int bt;
+        size_t bl;
+        unsigned bg;
+        if (make_tile_args(g, numActive, vec, b, bt, bl, bg, 24 * 1024) && b.psplit < a.psplit) {
+            a = b;
+            threads = bt;
+            ldsBytes = bl;
+            grid = bg;
+        }
+    }
+    return true;
+}
+
+template <typename G>
+static bool tile_match(const TileArgs& a, int threads)
+{
+    return !a.g.forceGeneric && a.g.R * a.g.S == (int)G::kRS && a.g.S == (int)G::S(a) && a.g.C == (int)G::C(a) &&
+           a.P == (int)G::P(a) && a.psplit == (int)G::kPsplit && threads == (int)G::nthr(a) && a.Pp == (int)G::kPp &&
+           a.Ct == (int)G::Ct(a) && a.lppLog == (int)G::kLppLog && a.vpr == G::kVpr && a.tpb == G::tpb(a);
+}
+
+template <int VEC, int MODE, typename G>
+static bool launch_fixed_scatter_one(const float* x, float* y, const float* ysrc, const int16_t* idx, const TileArgs& a,
+                                     int threads, size_t lds, int numActive, const ColorArgs& aux, hipStream_t stream)
+{
+    if (!tile_match<G>(a, threads)) return false;
+    hipLaunchKernelGGL((k_scatter_planar<VEC, MODE, G>), tile_grid(a.grid2d, a.tpb, numActive, a.total, a.g), dim3(threads),
+                       lds, stream, x, y, ysrc, idx, a, aux);
+    return true;
+}
+
+template <int VEC, int MODE>
+static bool launch_fixed_scatter(const float* x, float* y, const float* ysrc, const int16_t* idx, const TileArgs& a,
+                                 int threads, size_t lds, int numActive, const ColorArgs& aux, hipStream_t stream)
+{
+    if constexpr (VEC == 4 && (MODE == SCATTER_ASSIGN || MODE == SCATTER_ADD || MODE == SCATTER_RANKED)) {
+        // 27x27 blocks of 128 channels with 16 KB and 24 KB tiles; 16x16 blocks of 64 channels
+        return launch_fixed_scatter_one<VEC, MODE, TileFixed<27, 27, 128, 124, 512>>(x, y, ysrc, idx, a, threads, lds,
+                                                                                      numActive, aux, stream) ||
+               launch_fixed_scatter_one<VEC, MODE, TileFixed<27, 27, 128, 184, 512>>(x, y, ysrc, idx, a, threads, lds,
+                                                                                      numActive, aux, stream) ||
+               launch_fixed_scatter_one<VEC, MODE, TileFixed<16, 16, 64, 128, 512>>(x, y, ysrc, idx, a, threads, lds,
+                                                                                     numActive, aux, stream);
+    }
+    return false;
+}
+
+// The scatter's half of the tile_choice test hook (kind 2): same `out` fields.
+int scatter_tile_choice(const Geom& g, int numActive, int vec, int32_t* out)
+{
+    int threads = 0;
+    size_t lds = 0;
+    unsigned grid = 0;
+    const int RS = g.R * g.S;
+    TileArgs a;
+    if (RS < 4 || !scatter_tile_args(g, numActive, vec, a, threads, lds, grid)) return 0;
+    const int lpp = 1 << a.lppLog;
+    out[0] = threads; out[1] = (int32_t)lds; out[2] = a.P; out[3] = a.Pp; out[4] = a.psplit; out[5] = a.Ct;
+    out[6] = a.cchunks;
+    // per thread: NHWC items and planar slots of a full tile
+    const int items = (a.P * lpp + threads - 1) / threads;
+    const int slots = (int)((a.Ct * a.vpr + threads - 1) / threads);
+    out[7] = items > slots ? items : slots;
+    out[8] = TILE_LD;
+    out[9] = RS - (a.psplit - 1) * a.P;
+    out[10] = vec == 4 &&
+              (tile_match<TileFixed<27, 27, 128, 124, 512>>(a, threads) || tile_match<TileFixed<27, 27, 128, 184, 512>>(a, threads) ||
+               tile_match<TileFixed<16, 16, 64, 128, 512>>(a, threads));
+    return 1;
+}
+
+// `ysrc` is what an add reads: y itself for the in-place op, the base tensor when y is being built as
+// "copy of the base + scatter" without copying the covered pixels first.
+template <int VEC, int MODE>
+static void scatter_dispatch(const float* x, float* y, const float* ysrc, const int16_t* idx, const Geom& g,
+                             int numActive, bool transpose, hipStream_t stream, hipError_t& err,
+                             const int32_t* order = nullptr)
+{
+    // `order`: the owner map (SCATTER_OWNED) or the rank table (SCATTER_RANKED)
+    const ColorArgs aux{1, 1, 0, nullptr, MODE == SCATTER_OWNED ? order : nullptr,
+                        MODE == SCATTER_RANKED ? order : nullptr};
+    const int32_t* owner = order;
+    if (!transpose) {
+        NhwcArgs a;
+        if (!make_nhwc_args(g, numActive, VEC, a)) { err = hipErrorInvalidValue; return; }
+        if (nhwc_fits_buffers(g))
+            hipLaunchKernelGGL((k_scatter_nhwc<VEC, MODE>), dim3((a.units + 3) / 4), dim3(256), 0, stream, x, y, ysrc,
+                               idx, a, aux);
+        else
+            hipLaunchKernelGGL((k_scatter_nhwc_wide<VEC, MODE>), dim3((a.units + 3) / 4), dim3(256), 0, stream, x, y,
+                               ysrc, idx, a, aux);
+    } else {
+        TileArgs a;
+        int threads;
+        size_t lds;
+        unsigned grid;
+        // 16 KB tiles: 42.6 us against 43.9 us with 32 KB tiles on the same workload
+        if ((int64_t)g.R * g.S < 4 || !scatter_tile_args(g, numActive, VEC, a, threads, lds, grid)) {
+            const int64_t total = (int64_t)numActive * g.C * g.R * g.S;
+            const int64_t wgs = (total + 255) / 256;
+            hipLaunchKernelGGL((k_planar_small<MODE, false>), dim3((unsigned)(wgs > 65536 ? 65536 : wgs)), dim3(256),
+                               0, stream, x, y, ysrc, idx, g, total, owner);
+            return;
+        }
+        if (launch_fixed_scatter<VEC, MODE>(x, y, ysrc, idx, a, threads, lds, numActive, aux, stream)) return;
+        hipLaunchKernelGGL((k_scatter_planar<VEC, MODE, TileRt>), tile_grid(a.grid2d, a.tpb, numActive, a.total, a.g),
+                           dim3(threads), lds, stream, x, y, ysrc, idx, a, aux);
+    }
+}
+
+template <int VEC>
+static void scatter_mode(const float* x, float* y, const float* ysrc, const int16_t* idx, const Geom& g, int numActive,
+                         bool transpose, ScatterMode mode, hipStream_t stream, hipError_t& err, const int32_t* order,
+                         bool ranked)
+{
+    if (mode == SCATTER_ASSIGN && order && ranked)
+        scatter_dispatch<VEC, SCATTER_RANKED>(x, y, ysrc, idx, g, numActive, transpose, stream, err, order);
+    else if (mode == SCATTER_ASSIGN && order)
+        scatter_dispatch<VEC, SCATTER_OWNED>(x, y, ysrc, idx, g, numActive, transpose, stream, err, order);
+    else if (mode == SCATTER_ASSIGN)
+        scatter_dispatch<VEC, SCATTER_ASSIGN>(x, y, ysrc, idx, g, numActive, transpose, stream, err);
+    else if (mode == SCATTER_ADD)
+        scatter_dispatch<VEC, SCATTER_ADD>(x, y, ysrc, idx, g, numActive, transpose, stream, err);
+    else
+        scatter_dispatch<VEC, SCATTER_ATOMIC>(x, y, ysrc, idx, g, numActive, transpose, stream, err);
+}
+
+static hipError_t scatter_from(const float* x, float* y, const float* ysrc, const int16_t* idx, int numActive,
+                               const Geom& g, bool transpose, ScatterMode mode, hipStream_t stream,
+                               const int32_t* order = nullptr, bool ranked = false)
+{
+    if (numActive == 0) return hipSuccess;
+    hipError_t err = hipSuccess;
+    int vec = pick_vec(g, y, transpose ? nullptr : x);
+    const int vsrc = pick_vec(g, ysrc, nullptr);
+    if (vsrc < vec) vec = vsrc;
+    if (vec == 4) scatter_mode<4>(x, y, ysrc, idx, g, numActive, transpose, mode, stream, err, order, ranked);
+    else if (vec == 2) scatter_mode<2>(x, y, ysrc, idx, g, numActive, transpose, mode, stream, err, order, ranked);
+    else scatter_mode<1>(x, y, ysrc, idx, g, numActive, transpose, mode, stream, err, order, ranked);
+    if (err != hipSuccess) return err;
+    return hipGetLastError();
+}
+
+hipError_t launch_scatter(const float* x, float* y, const int16_t* idx, int numActive, const Geom& g,
+                          bool transpose, ScatterMode mode, hipStream_t stream)
+{
+    return scatter_from(x, y, y, idx, numActive, g, transpose, mode, stream);
+}
+
+// Extent of the inverse block map (blocks that can touch the image); false when it cannot be built.
+static bool make_map_args(const Geom& g, PullArgs& a, int64_t& mapN)
+{
+    a.g = g;
+    // oh + bh*U + R - 1 >= 0 and oh + bh*U <= H - 1 (floor divisions)
+    auto floordiv = [](int64_t p, int64_t q) { return p >= 0 ? p / q : -((-p + q - 1) / q); };
+    int64_t bhMin = -floordiv((int64_t)g.R - 1 + g.oh, g.U), bhMax = floordiv((int64_t)g.H - 1 - g.oh, g.U);
+    int64_t bwMin = -floordiv((int64_t)g.S - 1 + g.ow, g.V), bwMax = floordiv((int64_t)g.W - 1 - g.ow, g.V);
+    if (bhMin < -32768) bhMin = -32768;
+    if (bwMin < -32768) bwMin = -32768;
+    if (bhMax > 32767) bhMax = 32767;
+    if (bwMax > 32767) bwMax = 32767;
+    if (bhMax < bhMin || bwMax < bwMin) return false;
+    a.bhMin = (int)bhMin; a.bwMin = (int)bwMin;
+    a.nBH = (int)(bhMax - bhMin + 1); a.nBW = (int)(bwMax - bwMin + 1);
+    mapN = (int64_t)g.N * a.nBH * a.nBW;
+    return mapN < (1ll << 31);
+}
+
+// Geometry of the pull scatter; false when the method does not apply.
+static bool make_pull_args(const Geom& g, int numActive, int vec, PullArgs& a, int64_t& mapN)
+{
+    const int Kh = (g.R + g.U - 1) / g.U, Kw = (g.S + g.V - 1) / g.V;
+    if (Kh > 2 || Kw > 2) return false;  // at most 2x2 blocks over a pixel: neighbours one step away only
+    if (!make_map_args(g, a, mapN)) return false;
+    a.kh1 = Kh - 1;
+    a.kw1 = Kw - 1;
+    const uint64_t rowV = (uint64_t)g.S * g.C / vec, blockV = rowV * g.R;
+    if (blockV >= (1ull << 31)) return false;
+    a.CV = (uint32_t)(g.C / vec);
+    a.rowV = (uint32_t)rowV;
+    a.blockV = (uint32_t)blockV;
+    a.cpb = (uint32_t)((blockV + 64 * PULL_STEPS - 1) / (64 * PULL_STEPS));
+    const uint64_t units = (uint64_t)numActive * a.cpb;
+    if (units >= (1ull << 31)) return false;
+    a.units = (uint32_t)units;
+    a.dCpb = make_fastdiv(a.cpb);
+    a.dRow = make_fastdiv(a.rowV);
+    a.dCV = make_fastdiv(a.CV);
+    return true;
+}
+
+size_t scatter_pull_workspace_bytes(const Geom& g, int numActive)
+{
+    PullArgs a;
+    int64_t mapN = 0;
+    if (numActive <= 0 || !make_pull_args(g, numActive, 1, a, mapN)) return 0;
+    return (size_t)mapN * 4 + 16 + 16 + (size_t)numActive * PULL_TABLE_STRIDE * 4;  // map, flag, alignment, table
+}
+
+hipError_t launch_scatter_pull(const float* x, float* y, const int16_t* idx, int numActive, const Geom& g,
+                               void* workspace, size_t workspaceBytes, hipStream_t stream, bool& done)
+{
+    done = false;
+    if (numActive == 0) { done = true; return hipSuccess; }
+    PullArgs a;
+    int64_t mapN = 0;
+    const int vec = pick_vec(g, y, x);
+    if (!workspace || !make_pull_args(g, numActive, vec, a, mapN)) return hipSuccess;
+    if (workspaceBytes < scatter_pull_workspace_bytes(g, numActive) || (reinterpret_cast<uintptr_t>(workspace) & 3))
+        return hipSuccess;
+    int32_t* map = static_cast<int32_t*>(workspace);
+    int32_t* dup = map + mapN;
+    // the table is read with 16-byte loads
+    int32_t* table = reinterpret_cast<int32_t*>((reinterpret_cast<uintptr_t>(dup + 4) + 15) & ~(uintptr_t)15);
+    int64_t fillWgs = (mapN + 255) / 256;
+    if (fillWgs > 4096) fillWgs = 4096;
+    if (fillWgs < 1) fillWgs = 1;
+    const unsigned perBlockWgs = (unsigned)((numActive + 255) / 256);
+    hipLaunchKernelGGL(k_pull_fill, dim3((unsigned)fillWgs), dim3(256), 0, stream, map, mapN, dup);
+    hipLaunchKernelGGL(k_pull_map, dim3(perBlockWgs), dim3(256), 0, stream, idx, numActive, a, map, dup);
+    hipLaunchKernelGGL(k_pull_table, dim3((unsigned)(((int64_t)numActive * PULL_CLASSES + 255) / 256)), dim3(256), 0,
+                       stream, idx, numActive, a, map, table);
+    const unsigned wgs = (a.units + 3) / 4;
+    if (vec == 4) hipLaunchKernelGGL(k_scatter_pull<4>, dim3(wgs), dim3(256), 0, stream, x, y, idx, a, table, dup);
+    else if (vec == 2) hipLaunchKernelGGL(k_scatter_pull<2>, dim3(wgs), dim3(256), 0, stream, x, y, idx, a, table, dup);
+    else hipLaunchKernelGGL(k_scatter_pull<1>, dim3(wgs), dim3(256), 0, stream, x, y, idx, a, table, dup);
+    done = true;
+    return hipGetLastError();
+}
+
+// ---- scatter-add in passes ------------------------------------------------------------------
+
+constexpr int COLOR_MAX_PASSES = 16;
+
+size_t scatter_color_workspace_bytes(const Geom& g, int numActive)
+{
+    PullArgs a;
+    int64_t mapN = 0;
+    const int64_t Kh = ((int64_t)g.R + g.U - 1) / g.U, Kw = ((int64_t)g.S + g.V - 1) / g.V;
+    if (numActive <= 0 || Kh * Kw > COLOR_MAX_PASSES || !make_map_args(g, a, mapN)) return 0;
+    return (size_t)mapN * 4 + 16;
+}
+
+template <int VEC>
+static bool color_passes(const float* x, float* y, const int16_t* idx, const Geom& g, int numActive, bool transpose,
+                         ColorArgs col, int passes, hipStream_t stream)
+{
+    if (!transpose) {
+        NhwcArgs a;
+        if (!make_nhwc_args(g, numActive, VEC, a)) return false;
+        const bool buf = nhwc_fits_buffers(g);
+        for (col.pass = 0; col.pass < passes; ++col.pass) {
+            if (buf)
+                hipLaunchKernelGGL((k_scatter_nhwc<VEC, SCATTER_COLOR>), dim3((a.units + 3) / 4), dim3(256), 0, stream,
+                                   x, y, (const float*)y, idx, a, col);
+            else
+                hipLaunchKernelGGL((k_scatter_nhwc_wide<VEC, SCATTER_COLOR>), dim3((a.units + 3) / 4), dim3(256), 0,
+                                   stream, x, y, (const float*)y, idx, a, col);
+        }
+    } else {
+        TileArgs a;
+        int threads;
+        size_t lds;
+        unsigned grid;
+        if ((int64_t)g.R * g.S < 4 || !scatter_tile_args(g, numActive, VEC, a, threads, lds, grid, passes)) return false;
+        for (col.pass = 0; col.pass < passes; ++col.pass)
+            hipLaunchKernelGGL((k_scatter_planar<VEC, SCATTER_COLOR, TileRt>), tile_grid(a.grid2d, a.tpb, numActive, a.total, a.g),
+                               dim3(threads), lds, stream, x, y, (const float*)y, idx, a, col);
+    }
+    return true;
+}
+
+hipError_t launch_scatter_colored(const float* x, float* y, const int16_t* idx, int numActive, const Geom& g,
+                                  bool transpose, void* workspace, size_t workspaceBytes, hipStream_t stream,
+                                  bool& done)
+{
+    done = false;
+    if (numActive == 0) { done = true; return hipSuccess; }
+    const size_t need = scatter_color_workspace_bytes(g, numActive);
+    if (!workspace || need == 0 || workspaceBytes < need || (reinterpret_cast<uintptr_t>(workspace) & 3))
+        return hipSuccess;
+    PullArgs pa;
+    int64_t mapN = 0;
+    if (!make_map_args(g, pa, mapN)) return hipSuccess;
+    ColorArgs col;
+    col.kh = (g.R + g.U - 1) / g.U;
+    col.kw = (g.S + g.V - 1) / g.V;
+    col.pass = 0;
+    int32_t* map = static_cast<int32_t*>(workspace);
+    int32_t* dup = map + mapN;
+    col.dup = dup;
+    // geometry checks first: nothing is launched unless the passes can run
+    const int vec = pick_vec(g, y, transpose ? nullptr : x);
+    {
+        NhwcArgs na;
+        TileArgs ta;
+        int threads;
+        size_t lds;
+        unsigned grid;
+        if (!transpose ? !make_nhwc_args(g, numActive, vec, na)
+                       : ((int64_t)g.R * g.S < 4 || !scatter_tile_args(g, numActive, vec, ta, threads, lds, grid, col.kh * col.kw)))
+            return hipSuccess;
+    }
+    int64_t fillWgs = (mapN + 255) / 256;
+    if (fillWgs > 4096) fillWgs = 4096;
+    if (fillWgs < 1) fillWgs = 1;
+    hipLaunchKernelGGL(k_pull_fill, dim3((unsigned)fillWgs), dim3(256), 0, stream, map, mapN, dup);
+    hipLaunchKernelGGL(k_pull_map, dim3((unsigned)((numActive + 255) / 256)), dim3(256), 0, stream, idx, numActive, pa,
+                       map, dup);
+    const int passes = col.kh * col.kw;
+    if (vec == 4) color_passes<4>(x, y, idx, g, numActive, transpose, col, passes, stream);
+    else if (vec == 2) color_passes<2>(x, y, idx, g, numActive, transpose, col, passes, stream);
+    else color_passes<1>(x, y, idx, g, numActive, transpose, col, passes, stream);
+    done = true;
+    return hipGetLastError();
+}
+
+// ---- "copy of the base + scatter" without copying what the scatter overwrites -------------------
+//
+// sparse_scatter (not the in-place op) returns a fresh tensor: the base, with the blocks written or added on
+// top (sparse_gather.cc:338-346 copies the whole base, then scatters).  Copy-then-scatter moves every
+// covered pixel twice more than needed.  With one flag byte per pixel ("an active block covers it") the work
+// splits into two disjoint parts: k_copy_uncovered copies the pixels without the flag, and the ordinary
+// scatter kernels write the flagged ones, reading the base (`ysrc`) where they add.  Same result, every byte
+// moved once.  The flags cost N*H*W bytes of scratch and two small launches (clear, mark).
+
+struct CoverArgs {
+    Geom g;
+    uint32_t RS;
+    uint32_t imgV;      // vectors per image
+    uint32_t imgBytes;
+    int64_t imgFloats, imgPixels;
+    FastDiv dCV, dS;
+};
+
+constexpr int COVER_UNR = 4;
+
+__global__ __launch_bounds__(256) void k_cover_clear(uint32_t* __restrict__ words, int64_t n)
+{
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) words[i] = 0u;
+}
+
+// One thread per (block, block pixel): flags the pixel if it lies inside the image.  Blocks past the device-
+// resident count and rows with an image number outside [0, N) flag nothing, as they scatter nothing.
+__global__ __launch_bounds__(256) void k_cover_mark(const int16_t* __restrict__ idx, int numActive, CoverArgs a,
+                                                    uint8_t* __restrict__ flags)
+{
+    const int64_t total = (int64_t)numActive * a.RS;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const uint32_t ib = (uint32_t)(i / a.RS);
+        if (a.g.countDev && ib >= (uint32_t)*a.g.countDev) return;
+        const uint32_t p = (uint32_t)(i - (int64_t)ib * a.RS);
+        const uint32_t r = fdiv(p, a.dS), sc = p - r * (uint32_t)a.g.S;
+        const BlockOrigin o = load_origin(idx, ib, a.g);
+        const int hh = o.h0 + (int)r, ww = o.w0 + (int)sc;
+        if (o.valid && (unsigned)hh < (unsigned)a.g.H && (unsigned)ww < (unsigned)a.g.W)
+            flags[(int64_t)o.n * a.imgPixels + (int64_t)hh * a.g.W + ww] = 1;
+    }
+}
+
+// Owner map of the ordered plain scatter (SCATTER_OWNED): -1 everywhere, then the highest list position among the
+// blocks that cover each pixel.  Rows past the device-resident count and rows that name no image mark nothing.
+__global__ __launch_bounds__(256) void k_owner_fill(int32_t* __restrict__ owner, int64_t n)
+{
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) owner[i] = -1;
+}
+
+__global__ __launch_bounds__(256) void k_owner_mark(const int16_t* __restrict__ idx, int numActive, CoverArgs a,
+                                                    int32_t* __restrict__ owner)
+{
+    const int64_t total = (int64_t)numActive * a.RS;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const uint32_t ib = (uint32_t)(i / a.RS);
+        if (a.g.countDev && ib >= (uint32_t)*a.g.countDev) return;
+        const uint32_t p = (uint32_t)(i - (int64_t)ib * a.RS);
+        const uint32_t r = fdiv(p, a.dS), sc = p - r * (uint32_t)a.g.S;
+        const BlockOrigin o = load_origin(idx, ib, a.g);
+        const int hh = o.h0 + (int)r, ww = o.w0 + (int)sc;
+        if (o.valid && (unsigned)hh < (unsigned)a.g.H && (unsigned)ww < (unsigned)a.g.W)
+            atomicMax(owner + ((int64_t)o.n * a.imgPixels + (int64_t)hh * a.g.W + ww), (int32_t)ib);
+    }
+}
+
+// FLAG is the per-pixel coverage record: one byte (non-zero = covered), or the int32 owner map (>= 0 = covered).
+template <int VEC, typename FLAG>
+__global__ __launch_bounds__(256) void k_copy_uncovered(const float* __restrict__ src, float* __restrict__ dst,
+                                                        const FLAG* __restrict__ flags, CoverArgs a)
+{
+    typedef typename Vec<VEC>::type vec;
+    const uint32_t n = blockIdx.y;
+    const rsrc_t sr = make_rsrc(src + (int64_t)n * a.imgFloats, a.imgBytes);
+    const rsrc_t dr = make_rsrc(dst + (int64_t)n * a.imgFloats, a.imgBytes);
+    const FLAG* __restrict__ fl = flags + (int64_t)n * a.imgPixels;
+    const uint32_t e0 = blockIdx.x * (256u * COVER_UNR) + threadIdx.x;
+    bool cov[COVER_UNR];
+#pragma unroll
+    for (int u = 0; u < COVER_UNR; ++u) {
+        const uint32_t e = min(e0 + (uint32_t)u * 256u, a.imgV - 1u);
+        const FLAG f = fl[fdiv(e, a.dCV)];
+        cov[u] = sizeof(FLAG) == 1 ? f != 0 : (int32_t)f >= 0;
+    }
+    uint32_t off[COVER_UNR];
+#pragma unroll
+    for (int u = 0; u < COVER_UNR; ++u) {
+        const uint32_t e = e0 + (uint32_t)u * 256u;
+        off[u] = (e >= a.imgV || cov[u]) ? BUF_OOB : e * (uint32_t)(VEC * 4);
+    }
+    vec v[COVER_UNR];
+#pragma unroll
+    for (int u = 0; u < COVER_UNR; ++u) v[u] = buf_load<VEC>(sr, off[u]);
+#pragma unroll
+    for (int u = 0; u < COVER_UNR; ++u) buf_store<BUF_NT>(dr, off[u], v[u]);
+}
+
+size_t scatter_cover_workspace_bytes(const Geom& g, int numActive)
+{
+    if (numActive <= 0) return 0;
+    if ((int64_t)g.H * g.W * g.C >= (1ll << 30)) return 0;  // 32-bit byte offsets inside one image
+    if ((int64_t)g.R * g.S >= (1ll << 31)) return 0;
+    return (((size_t)g.N * g.H * g.W + 3) & ~(size_t)3) + 16;
+}
+
+static void make_cover_args(const Geom& g, int vec, CoverArgs& c)
+{
+    c.g = g;
+    c.RS = (uint32_t)(g.R * g.S);
+    c.imgFloats = (int64_t)g.H * g.W * g.C;
+    c.imgPixels = (int64_t)g.H * g.W;
+    c.imgV = (uint32_t)(c.imgFloats / vec);
+    c.imgBytes = (uint32_t)(c.imgFloats * 4);
+    c.dCV = make_fastdiv((uint32_t)(g.C / vec));
+    c.dS = make_fastdiv((uint32_t)g.S);
+}
+
+// Nine bits per block for SCATTER_RANKED.  One wave per block: the lanes compare the block with every row of the
+// list; a later row that names the same image and a grid position within one step in both directions sets the
+// classes of pixels it shares with the block (itself included: a block listed twice loses all its pixels to the
+// later row).
+constexpr int RANK_MAX_BLOCKS = 4096;   // rows compared pairwise: 16.8 M comparisons at most
+
+__global__ __launch_bounds__(256) void k_rank_table(const int16_t* __restrict__ idx, int numActive, Geom g,
+                                                    int32_t* __restrict__ table)
+{
+    const uint32_t lane = threadIdx.x & 63u;
+    const int ib = (int)(blockIdx.x * 4u + (threadIdx.x >> 6));
+    int count = numActive;
+    if (g.countDev) count = min(count, *g.countDev);
+    if (ib >= count) return;
+    const int n = idx[(size_t)ib * 3], bh = idx[(size_t)ib * 3 + 1], bw = idx[(size_t)ib * 3 + 2];
+    uint32_t bits = 0u;
+    for (int j = ib + 1 + (int)lane; j < count; j += 64) {
+        const int dn = idx[(size_t)j * 3] - n, dh = idx[(size_t)j * 3 + 1] - bh, dw = idx[(size_t)j * 3 + 2] - bw;
+        if (dn == 0 && dh >= -1 && dh <= 1 && dw >= -1 && dw <= 1) {
+            // row classes (0: first R-U rows, 1: middle, 2: rows from U on) that a block dh steps away covers
+            const uint32_t rows = dh < 0 ? 1u : (dh > 0 ? 4u : 7u), cols = dw < 0 ? 1u : (dw > 0 ? 4u : 7u);
+#pragma unroll
+            for (int rc = 0; rc < 3; ++rc)
+                if (rows & (1u << rc)) bits |= cols << (3 * rc);
+        }
+    }
+    for (int off = 32; off > 0; off >>= 1) bits |= (uint32_t)__shfl_xor((int)bits, off);
+    if (lane == 0) table[ib] = (int32_t)bits;
+}
+
+// The rank table applies when at most 2x2 blocks share a pixel and the list is short enough for pairwise comparison.
+static bool rank_table_applies(const Geom& g, int numActive)
+{
+    return numActive <= RANK_MAX_BLOCKS && g.R <= 2 * (int64_t)g.U && g.S <= 2 * (int64_t)g.V;
+}
+
+size_t scatter_owner_workspace_bytes(const Geom& g, int numActive)
+{
+    if (numActive <= 0 || !(g.U < g.R || g.V < g.S)) return 0;  // only overlapping blocks need an order
+    if ((int64_t)g.R * g.S >= (1ll << 31)) return 0;
+    // (the owner map; the rank table of the in-place op needs less, but the copying op always takes the map)
+    const size_t map = (size_t)g.N * g.H * g.W * 4 + 16, table = (size_t)numActive * 4 + 16;
+    return map > table ? map : table;
+}
+
+// Builds the owner map in `workspace`; false (nothing launched) when the ordered scatter does not apply.
+static bool build_owner_map(const int16_t* idx, int numActive, const Geom& g, void* workspace, size_t workspaceBytes,
+                            hipStream_t stream, int32_t*& owner)
+{
+    const size_t need = scatter_owner_workspace_bytes(g, numActive);
+    if (!workspace || need == 0 || workspaceBytes < need || (reinterpret_cast<uintptr_t>(workspace) & 3)) return false;
+    owner = static_cast<int32_t*>(workspace);
+    CoverArgs c;
+    make_cover_args(g, 1, c);
+    const int64_t n = (int64_t)g.N * g.H * g.W;
+    int64_t wgs = (n + 1023) / 1024;
+    if (wgs > 8192) wgs = 8192;
+    hipLaunchKernelGGL(k_owner_fill, dim3((unsigned)wgs), dim3(256), 0, stream, owner, n);
+    int64_t markWgs = ((int64_t)numActive * c.RS + 255) / 256;
+    if (markWgs > 65536) markWgs = 65536;
+    hipLaunchKernelGGL(k_owner_mark, dim3((unsigned)markWgs), dim3(256), 0, stream, idx, numActive, c, owner);
+    return true;
+}
+
+hipError_t launch_scatter_owned(const float* x, float* y, const int16_t* idx, int numActive, const Geom& g,
+                                bool transpose, void* workspace, size_t workspaceBytes, hipStream_t stream, bool& done)
+{
+    done = false;
+    if (numActive == 0) { done = true; return hipSuccess; }
+    if (rank_table_applies(g, numActive) && scatter_owner_workspace_bytes(g, numActive) != 0 && workspace &&
+        workspaceBytes >= (size_t)numActive * 4 + 16 && (reinterpret_cast<uintptr_t>(workspace) & 3) == 0) {
+        int32_t* table = static_cast<int32_t*>(workspace);
+        hipLaunchKernelGGL(k_rank_table, dim3((unsigned)((numActive + 3) / 4)), dim3(256), 0, stream, idx, numActive, g,
+                           table);
+        done = true;
+        return scatter_from(x, y, y, idx, numActive, g, transpose, SCATTER_ASSIGN, stream, table, true);
+    }
+    int32_t* owner = nullptr;
+    if (!build_owner_map(idx, numActive, g, workspace, workspaceBytes, stream, owner)) return hipSuccess;
+    done = true;
+    return scatter_from(x, y, y, idx, numActive, g, transpose, SCATTER_ASSIGN, stream, owner);
+}
+
+hipError_t launch_scatter_over_base(const float* x, const float* ybase, float* y, const int16_t* idx, int numActive,
+                                    const Geom& g, bool transpose, ScatterMode mode, void* workspace,
+                                    size_t workspaceBytes, hipStream_t stream, bool& done)
+{
+    done = false;
+    if (mode == SCATTER_ATOMIC || numActive <= 0) return hipSuccess;
+    const size_t need = scatter_cover_workspace_bytes(g, numActive);
+    if (!workspace || need == 0 || workspaceBytes < need || (reinterpret_cast<uintptr_t>(workspace) & 3))
+        return hipSuccess;
+    // Two small launches prepare the flags: worth it once the blocks cover enough of the tensor to pay for them
+    // (each covered byte saves one read and one write of the copy).
+    if ((int64_t)numActive * g.R * g.S * g.C * 4 < (16ll << 20)) return hipSuccess;
+
+    CoverArgs c;
+    const int vec = pick_vec(g, ybase, y);
+    make_cover_args(g, vec, c);
+    const dim3 grid((c.imgV + 256u * COVER_UNR - 1) / (256u * COVER_UNR), (unsigned)g.N);
+
+    // Plain writes of overlapping blocks: the owner map of the ordered scatter also tells which pixels are covered.
+    if (mode == SCATTER_ASSIGN && scatter_owner_workspace_bytes(g, numActive) != 0) {
+        int32_t* owner = nullptr;
+        if (!build_owner_map(idx, numActive, g, workspace, workspaceBytes, stream, owner)) return hipSuccess;
+        if (vec == 4) hipLaunchKernelGGL((k_copy_uncovered<4, int32_t>), grid, dim3(256), 0, stream, ybase, y, owner, c);
+        else if (vec == 2) hipLaunchKernelGGL((k_copy_uncovered<2, int32_t>), grid, dim3(256), 0, stream, ybase, y, owner, c);
+        else hipLaunchKernelGGL((k_copy_uncovered<1, int32_t>), grid, dim3(256), 0, stream, ybase, y, owner, c);
+        done = true;
+        return scatter_from(x, y, ybase, idx, numActive, g, transpose, mode, stream, owner);
+    }
+    uint8_t* flags = static_cast<uint8_t*>(workspace);
+
+    const int64_t words = (int64_t)((need - 16) / 4);
+    int64_t wgs = (words + 255) / 256;
+    if (wgs > 8192) wgs = 8192;
+    hipLaunchKernelGGL(k_cover_clear, dim3((unsigned)wgs), dim3(256), 0, stream, reinterpret_cast<uint32_t*>(flags), words);
+    int64_t markWgs = ((int64_t)numActive * c.RS + 255) / 256;
+    if (markWgs > 65536) markWgs = 65536;
+    hipLaunchKernelGGL(k_cover_mark, dim3((unsigned)markWgs), dim3(256), 0, stream, idx, numActive, c, flags);
+    const uint8_t* cflags = flags;
+    if (vec == 4) hipLaunchKernelGGL((k_copy_uncovered<4, uint8_t>), grid, dim3(256), 0, stream, ybase, y, cflags, c);
+    else if (vec == 2) hipLaunchKernelGGL((k_copy_uncovered<2, uint8_t>), grid, dim3(256), 0, stream, ybase, y, cflags, c);
+    else hipLaunchKernelGGL((k_copy_uncovered<1, uint8_t>), grid, dim3(256), 0, stream, ybase, y, cflags, c);
+    done = true;
+    return scatter_from(x, y, ybase, idx, numActive, g, transpose, mode, stream);
+}
+
+hipError_t launch_copy(float* dst, const float* src, size_t count, hipStream_t stream)
+{
+    if (count == 0) return hipSuccess;
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src);
+    if ((bits & 15) == 0) {
+        const size_t n4 = count / 4;
+        if (n4) {
+            const size_t per = 256 * COPY_UNR;
+            hipLaunchKernelGGL(k_copy_v4, dim3((unsigned)((n4 + per - 1) / per)), dim3(256), 0, stream,
+                               reinterpret_cast<const f4*>(src), reinterpret_cast<f4*>(dst), n4);
+        }
+        const size_t rem = count - n4 * 4;
+        if (rem) hipLaunchKernelGGL(k_copy_scalar, dim3(1), dim3(256), 0, stream, src + n4 * 4, dst + n4 * 4, rem);
+    } else {
+        size_t wgs = (count + 255) / 256;
+        if (wgs > 65536) wgs = 65536;
+        hipLaunchKernelGGL(k_copy_scalar, dim3((unsigned)wgs), dim3(256), 0, stream, src, dst, count);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace sbnet
