@@ -377,16 +377,19 @@ def cpu_baseline(wl, M, idx_host, nbytes, budget_s=12.0):
 
 
 def kernel_source_digest():
-    """sha256 over the device sources the library is built from (csrc/*.hip and csrc/*.h, by name): the counters
-    under profiles/ belong to one state of them."""
+    """sha256 over the code of the device sources the library is built from (csrc/*.hip and csrc/*.h, by name,
+    comments and white space left out): the counters under profiles/ belong to one state of it."""
     import glob
     import hashlib
+    import re
     d = os.path.join(ROOT, "sbnet_amd", "csrc")
     h = hashlib.sha256()
     for p in sorted(glob.glob(os.path.join(d, "*.hip")) + glob.glob(os.path.join(d, "*.h"))):
-        h.update(os.path.basename(p).encode() + b"\0")
-        with open(p, "rb") as f:
-            h.update(f.read())
+        with open(p, "r") as f:
+            text = f.read()
+        text = re.sub(r"/\*.*?\*/", " ", text, flags=re.S)
+        text = re.sub(r"//[^\n]*", " ", text)      # (no string literal in these files holds "//")
+        h.update(os.path.basename(p).encode() + b"\0" + " ".join(text.split()).encode() + b"\0")
     return h.hexdigest()
 
 

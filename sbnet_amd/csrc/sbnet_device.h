@@ -430,8 +430,9 @@ template <int AUX> __device__ __forceinline__ void buf_store(rsrc_t r, uint32_t 
 
 // ---- NHWC stack <-> NHWC tensor with buffer addressing ------------------------------------------
 //
-// The row-segment copies again, for images and blocks below 2^30 floats (everything but the largest
-// tensors; the kernels above remain for those): both sides go through range-checked descriptors, lanes
+// k_gather_nhwc and k_scatter_nhwc are the row-segment copies for images and blocks below 2^30 floats
+// (everything but the largest tensors; the _wide kernels, with 64-bit addresses and branches, remain for
+// those): both sides go through range-checked descriptors, lanes
 // with nothing to move get an out-of-range offset, and there is no control flow between the first load
 // and the last store.  In the branchy version every conditional store was preceded by a full wait for
 // outstanding memory operations, stores included, so the four stores of a lane went out one after the

@@ -28,7 +28,10 @@ def test_kernel_digest_follows_the_sources(tmp_path, monkeypatch):
     monkeypatch.setattr(bench, "ROOT", str(tmp_path))
     assert bench.kernel_source_digest() == d0
     with open(csrc / "sbnet_launch.h", "ab") as f:
-        f.write(b"\n// changed\n")
+        f.write(b"\n// a comment   and /* another */\n\n")
+    assert bench.kernel_source_digest() == d0     # comments and white space are not code
+    with open(csrc / "sbnet_launch.h", "ab") as f:
+        f.write(b"\nconstexpr int changed = 1;\n")
     assert bench.kernel_source_digest() != d0
 
 
