@@ -267,8 +267,9 @@ int scatter_impl(const float* x, int32_t numActive, const int32_t* countDev, con
                                                 stream, done));
         if (done) return SBNET_OK;
     }
-    if (mode == sbnet::SCATTER_ASSIGN && workspace) {
-        // with scratch, overlapping plain writes land in the CPU functor's order (the block listed last wins)
+    if (mode == sbnet::SCATTER_ASSIGN) {
+        // overlapping plain writes land in the CPU functor's order (the block listed last wins): decided inside the
+        // planar kernel where that applies, else with scratch (nothing is done here without scratch then)
         bool done = false;
         SBNET_HIP(sbnet::launch_scatter_owned(x, out, idx, numActive, g, transpose != 0, workspace, workspaceBytes,
                                               stream, done));

@@ -200,6 +200,13 @@ constexpr int SCATTER_OWNED = 4;  // kernel-side mode; callers ask for SCATTER_A
 // later covers that class of pixels; the scatter kernels skip those pixels.
 constexpr int SCATTER_RANKED = 5;  // kernel-side mode; callers ask for SCATTER_ASSIGN and give scratch
 
+// The same nine bits without a table and without an extra launch: the workgroup that moves a tile of block ib
+// compares ib with the rows listed after it while the tile's loads are in flight (a few hundred 6-byte rows from
+// L2 against a 16-24 KB tile), so the in-place op needs neither scratch nor a second kernel for the CPU functor's
+// order.  Planar tile kernel only: its workgroups are large enough to share the comparison.
+constexpr int SCATTER_RANKED_INLINE = 6;  // kernel-side mode; callers ask for SCATTER_ASSIGN
+constexpr int RANK_ROWS_PER_THREAD = 2;   // rows of the list fetched per thread ahead of the tile's LDS phase
+
 struct ColorArgs {
     int kh, kw, pass;
     const int32_t* dup;
@@ -213,6 +220,25 @@ __device__ __forceinline__ bool ranked_out(uint32_t bits, uint32_t r, uint32_t s
     const uint32_t rc = (int)r < g.R - g.U ? 0u : ((int)r >= g.U ? 2u : 1u);
     const uint32_t cc = (int)s < g.S - g.V ? 0u : ((int)s >= g.V ? 2u : 1u);
     return (bits >> (rc * 3u + cc)) & 1u;
+}
+
+// Classes of block (n, bh, bw)'s pixels that the block of a later row (n2, bh2, bw2) covers: row classes (0: first
+// R-U rows, 1: middle, 2: rows from U on) crossed with the same for columns, bit 3*rowClass + colClass.
+__device__ __forceinline__ uint32_t rank_pair_bits(int n, int bh, int bw, int n2, int bh2, int bw2)
+{
+    const int dh = bh2 - bh, dw = bw2 - bw;
+    if (n2 != n || dh < -1 || dh > 1 || dw < -1 || dw > 1) return 0u;
+    const uint32_t rows = dh < 0 ? 1u : (dh > 0 ? 4u : 7u), cols = dw < 0 ? 1u : (dw > 0 ? 4u : 7u);
+    return ((rows & 1u) ? cols : 0u) | ((rows & 2u) ? cols << 3 : 0u) | ((rows & 4u) ? cols << 6 : 0u);
+}
+
+// Length of the block list as the kernels see it: the host's count, capped by the device-resident one.
+__device__ __forceinline__ uint32_t list_count(const Geom& g, uint32_t capacity)
+{
+    if (!g.countDev) return capacity;
+    typedef const int32_t __attribute__((address_space(4))) * const_i32_ptr;
+    const int32_t c = *(const_i32_ptr)(reinterpret_cast<uintptr_t>(g.countDev));
+    return min(capacity, (uint32_t)max(c, 0));
 }
 
 __device__ __forceinline__ uint32_t rank_bits(const ColorArgs& col, uint32_t ib)
@@ -415,6 +441,45 @@ template <> __device__ __forceinline__ float buf_load<1>(rsrc_t r, uint32_t off)
     return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, off, 0, 0));
 }
 
+// Rows of the block list through a buffer descriptor: row j is 6 bytes at 6*j, fetched as the two aligned dwords
+// around it with one 8-byte load (the descriptor starts at the list's address rounded down to 4 bytes and ends
+// with the aligned dword that holds the list's last int16, so the load of the last row stays inside it).
+struct ListRows {
+    rsrc_t r;
+    uint32_t mis;  // 0 or 2: the list's own misalignment
+};
+
+__device__ __forceinline__ ListRows list_rows(const int16_t* idx, uint32_t count)
+{
+    const uintptr_t p = reinterpret_cast<uintptr_t>(idx);
+    ListRows l;
+    l.mis = (uint32_t)(p & 2u);
+    l.r = make_rsrc(reinterpret_cast<const void*>(p & ~(uintptr_t)3), (l.mis + count * 6u + 3u) & ~3u);
+    return l;
+}
+
+struct ListRow {
+    u2 w;
+    uint32_t shift;  // 0 or 16
+};
+
+__device__ __forceinline__ ListRow list_row_load(const ListRows& l, uint32_t j, bool live)
+{
+    const uint32_t b = j * 6u + l.mis;
+    ListRow row;
+    row.w = __builtin_bit_cast(u2, __builtin_amdgcn_raw_buffer_load_b64(l.r, live ? (b & ~3u) : BUF_OOB, 0, 0));
+    row.shift = (b & 2u) * 8u;
+    return row;
+}
+
+__device__ __forceinline__ void list_row_unpack(const ListRow& row, int& n, int& bh, int& bw)
+{
+    const uint32_t nb = __builtin_amdgcn_alignbit(row.w.y, row.w.x, row.shift);  // (hi:lo) >> shift, low dword
+    n = (int)(int16_t)(nb & 0xffffu);
+    bh = (int)(int16_t)(nb >> 16);
+    bw = (int)(int16_t)(row.shift ? row.w.y >> 16 : row.w.y & 0xffffu);
+}
+
 template <int AUX> __device__ __forceinline__ void buf_store(rsrc_t r, uint32_t off, const f4& v)
 {
     __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4, v), r, off, 0, AUX);
@@ -523,7 +588,7 @@ __global__ __launch_bounds__(256) void k_planar_small(const float* __restrict__ 
                 if (owner[((int64_t)o.n * g.H + hh) * g.W + ww] == (int32_t)ib) y[pix] = x[st];
             } else if (MODE == SCATTER_RANKED) {
                 if (!ranked_out((uint32_t)owner[ib], (uint32_t)r, (uint32_t)s, g)) y[pix] = x[st];
-            } else if (MODE == SCATTER_ASSIGN) y[pix] = x[st];
+            } else if (MODE == SCATTER_ASSIGN || MODE == SCATTER_RANKED_INLINE) y[pix] = x[st];
             else if (MODE == SCATTER_ADD) y[pix] = ysrc[pix] + x[st];
             else atomic_add_f32(y + pix, x[st]);
         }

@@ -62,7 +62,8 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc_wide(const float* __restri
 #pragma unroll
         for (int u = 0; u < NHWC_UNR; ++u)
             if (dst[u] >= 0) st_stream(yv + dst[u], vadd(cur[u], v[u]));
-    } else if (MODE == SCATTER_ASSIGN || MODE == SCATTER_OWNED || MODE == SCATTER_RANKED) {
+    } else if (MODE == SCATTER_ASSIGN || MODE == SCATTER_OWNED || MODE == SCATTER_RANKED || MODE == SCATTER_RANKED_INLINE) {
+        // (SCATTER_RANKED_INLINE is never launched on this kernel; plain stores if it were)
 #pragma unroll
         for (int u = 0; u < NHWC_UNR; ++u)
             if (dst[u] >= 0) commit<VEC, SCATTER_ASSIGN>(yv + dst[u], v[u]);
@@ -123,7 +124,7 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
         // (an out-of-range owner read returns 0, which may equal ib: dst is BUF_OOB there already)
 #pragma unroll
         for (int u = 0; u < NHWC_UNR; ++u) buf_store<BUF_NT>(yr, own[u] == (int32_t)ib ? dst[u] : BUF_OOB, v[u]);
-    } else if (MODE == SCATTER_ASSIGN || MODE == SCATTER_RANKED) {
+    } else if (MODE == SCATTER_ASSIGN || MODE == SCATTER_RANKED || MODE == SCATTER_RANKED_INLINE) {
 #pragma unroll
         for (int u = 0; u < NHWC_UNR; ++u) buf_store<BUF_NT>(yr, dst[u], v[u]);
     } else if (MODE == SCATTER_ADD || (MODE == SCATTER_COLOR && !atomics)) {
@@ -148,7 +149,8 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
 template <int VEC, int MODE, typename G>
 __device__ __forceinline__ void scatter_planar_tile(const float* __restrict__ x, float* y, const float* ysrc,
                                                     const int16_t* __restrict__ idx, const TileArgs& a,
-                                                    const ColorArgs& col, float* lds, uint32_t ib, uint32_t rem)
+                                                    const ColorArgs& col, float* lds, uint32_t* waveBits,
+                                                    uint32_t ib, uint32_t rem)
 {
     typedef typename Vec<VEC>::type vec;
     const uint32_t tid = threadIdx.x, nthr = G::nthr(a);
@@ -165,6 +167,21 @@ __device__ __forceinline__ void scatter_planar_tile(const float* __restrict__ x,
     const rsrc_t xr = make_rsrc(x + ((int64_t)t.ib * G::C(a) + t.c0) * RS + t.p0,
                                 ((uint32_t)(t.ctEff - 1) * RS + (uint32_t)t.Pn) * 4u);
     const uint32_t slots = (uint32_t)t.ctEff * vpr;
+    // SCATTER_RANKED_INLINE: the rows listed after this block, RANK_ROWS_PER_THREAD per thread, fetched behind the
+    // tile's own loads (loads return in order, so they are there when the tile's data is)
+    ListRow rows[RANK_ROWS_PER_THREAD];
+    uint32_t listCount = 0;
+    ListRows lr;
+    auto fetch_rows = [&]() {
+        if (MODE != SCATTER_RANKED_INLINE) return;
+        listCount = list_count(a.g, a.blocks);
+        lr = list_rows(idx, listCount);
+#pragma unroll
+        for (int u = 0; u < RANK_ROWS_PER_THREAD; ++u) {
+            const uint32_t j = t.ib + 1u + (uint32_t)u * nthr + tid;
+            rows[u] = list_row_load(lr, j, j < listCount);
+        }
+    };
     if (t.Pn >= 4) {
         f4 val[TILE_LD];
 #pragma unroll
@@ -174,6 +191,7 @@ __device__ __forceinline__ void scatter_planar_tile(const float* __restrict__ x,
             const int e0 = min(4 * (int)(i - c * vpr), t.Pn - 4);
             val[u] = buf_load<4>(xr, i < slots ? (c * RS + (uint32_t)e0) * 4u : BUF_OOB);
         }
+        fetch_rows();
 #pragma unroll
         for (int u = 0; u < TILE_LD; ++u) {
             const uint32_t i = u * nthr + tid;
@@ -199,11 +217,32 @@ __device__ __forceinline__ void scatter_planar_tile(const float* __restrict__ x,
             for (int k = 0; k < t.Pn; ++k)
                 lds[tid * Pp + ((uint32_t)k ^ lds_swz(tid))] = buf_load<1>(xr, (tid * RS + (uint32_t)k) * 4u);
         }
+        fetch_rows();
+    }
+    const BlockOrigin o = origin_of(raw, a.g);
+    if (MODE == SCATTER_RANKED_INLINE) {
+        // nine bits: classes of this block's pixels that a block listed later covers (the later one wins them)
+        uint32_t bits = 0u;
+#pragma unroll
+        for (int u = 0; u < RANK_ROWS_PER_THREAD; ++u) {
+            int n2, bh2, bw2;
+            list_row_unpack(rows[u], n2, bh2, bw2);
+            if (t.ib + 1u + (uint32_t)u * nthr + tid < listCount) bits |= rank_pair_bits(o.n, o.bh, o.bw, n2, bh2, bw2);
+        }
+        // (lists with more than RANK_ROWS_PER_THREAD * nthr rows after this block)
+        for (uint32_t j = t.ib + 1u + (uint32_t)RANK_ROWS_PER_THREAD * nthr + tid; j < listCount; j += nthr) {
+            int n2, bh2, bw2;
+            list_row_unpack(list_row_load(lr, j, true), n2, bh2, bw2);
+            bits |= rank_pair_bits(o.n, o.bh, o.bw, n2, bh2, bw2);
+        }
+        // most waves see none of the few neighbouring rows
+        if (__ballot(bits != 0u) != 0ull)
+            for (int off = 32; off > 0; off >>= 1) bits |= (uint32_t)__shfl_xor((int)bits, off);
+        if ((tid & 63u) == 0u) waveBits[tid >> 6] = bits;
     }
     lds_barrier();
 
     // NHWC side: LDS -> base tensor; pixels outside the image are dropped (sparse_gather.cc:121)
-    const BlockOrigin o = origin_of(raw, a.g);
     if (!o.valid) return;
     float* img = y + (int64_t)o.n * a.imgFloats;
     const rsrc_t yr = make_rsrc(img, a.imgBytes);
@@ -214,9 +253,12 @@ __device__ __forceinline__ void scatter_planar_tile(const float* __restrict__ x,
     int32_t own[TILE_LD];
     const rsrc_t wr = make_rsrc(MODE == SCATTER_OWNED ? col.owner + (int64_t)o.n * a.g.H * a.g.W : nullptr,
                                 MODE == SCATTER_OWNED ? (uint32_t)(a.g.H * a.g.W) * 4u : 0u);
-    const uint32_t rbits = MODE == SCATTER_RANKED ? rank_bits(col, t.ib) : 0u;
+    uint32_t rbits = MODE == SCATTER_RANKED ? rank_bits(col, t.ib) : 0u;
+    if (MODE == SCATTER_RANKED_INLINE) {
+        for (uint32_t w = 0; w < (nthr >> 6); ++w) rbits |= waveBits[w];
+    }
     nhwc_walk<VEC, G>(a, t, o, tid, nthr, [&](int u, uint32_t pl, uint32_t off, uint32_t pix, uint32_t r, uint32_t sc) {
-        if (MODE == SCATTER_RANKED && ranked_out(rbits, r, sc, a.g)) off = BUF_OOB;
+        if ((MODE == SCATTER_RANKED || MODE == SCATTER_RANKED_INLINE) && ranked_out(rbits, r, sc, a.g)) off = BUF_OOB;
         offs[u] = off;
         if (MODE == SCATTER_OWNED) own[u] = __builtin_bit_cast(int32_t, buf_load<1>(wr, off != BUF_OOB ? pix * 4u : BUF_OOB));
         w[u] = vzero<VEC>();
@@ -231,7 +273,7 @@ __device__ __forceinline__ void scatter_planar_tile(const float* __restrict__ x,
     if (MODE == SCATTER_OWNED) {
 #pragma unroll
         for (int u = 0; u < TILE_LD; ++u) buf_store<BUF_NT>(yr, own[u] == (int32_t)t.ib ? offs[u] : BUF_OOB, w[u]);
-    } else if (MODE == SCATTER_ASSIGN || MODE == SCATTER_RANKED) {
+    } else if (MODE == SCATTER_ASSIGN || MODE == SCATTER_RANKED || MODE == SCATTER_RANKED_INLINE) {
 #pragma unroll
         for (int u = 0; u < TILE_LD; ++u) buf_store<BUF_NT>(yr, offs[u], w[u]);
     } else if (MODE == SCATTER_ADD || (MODE == SCATTER_COLOR && !atomics)) {
@@ -257,8 +299,9 @@ __global__ __launch_bounds__(512) void k_scatter_planar(const float* __restrict_
                                                         const int16_t* __restrict__ idx, TileArgs a, ColorArgs col)
 {
     extern __shared__ __attribute__((aligned(16))) float lds[];
+    __shared__ uint32_t waveBits[8];  // SCATTER_RANKED_INLINE: one word per wave
     for_each_block_of_workgroup(a, G::tpb(a), [&](uint32_t ib, uint32_t rem) {
-        scatter_planar_tile<VEC, MODE, G>(x, y, ysrc, idx, a, col, lds, ib, rem);
+        scatter_planar_tile<VEC, MODE, G>(x, y, ysrc, idx, a, col, lds, waveBits, ib, rem);
     });
 }
 
@@ -536,7 +579,8 @@ template <int VEC, int MODE>
 static bool launch_fixed_scatter(const float* x, float* y, const float* ysrc, const int16_t* idx, const TileArgs& a,
                                  int threads, size_t lds, int numActive, const ColorArgs& aux, hipStream_t stream)
 {
-    if constexpr (VEC == 4 && (MODE == SCATTER_ASSIGN || MODE == SCATTER_ADD || MODE == SCATTER_RANKED)) {
+    if constexpr (VEC == 4 && (MODE == SCATTER_ASSIGN || MODE == SCATTER_ADD || MODE == SCATTER_RANKED ||
+                               MODE == SCATTER_RANKED_INLINE)) {
         // 27x27 blocks of 128 channels with 16 KB and 24 KB tiles; 16x16 blocks of 64 channels
         return launch_fixed_scatter_one<VEC, MODE, TileFixed<27, 27, 128, 124, 512>>(x, y, ysrc, idx, a, threads, lds,
                                                                                       numActive, aux, stream) ||
@@ -614,9 +658,11 @@ static void scatter_dispatch(const float* x, float* y, const float* ysrc, const 
 template <int VEC>
 static void scatter_mode(const float* x, float* y, const float* ysrc, const int16_t* idx, const Geom& g, int numActive,
                          bool transpose, ScatterMode mode, hipStream_t stream, hipError_t& err, const int32_t* order,
-                         bool ranked)
+                         bool ranked, bool rankInline)
 {
-    if (mode == SCATTER_ASSIGN && order && ranked)
+    if (mode == SCATTER_ASSIGN && rankInline)
+        scatter_dispatch<VEC, SCATTER_RANKED_INLINE>(x, y, ysrc, idx, g, numActive, transpose, stream, err);
+    else if (mode == SCATTER_ASSIGN && order && ranked)
         scatter_dispatch<VEC, SCATTER_RANKED>(x, y, ysrc, idx, g, numActive, transpose, stream, err, order);
     else if (mode == SCATTER_ASSIGN && order)
         scatter_dispatch<VEC, SCATTER_OWNED>(x, y, ysrc, idx, g, numActive, transpose, stream, err, order);
@@ -630,16 +676,16 @@ static void scatter_mode(const float* x, float* y, const float* ysrc, const int1
 
 static hipError_t scatter_from(const float* x, float* y, const float* ysrc, const int16_t* idx, int numActive,
                                const Geom& g, bool transpose, ScatterMode mode, hipStream_t stream,
-                               const int32_t* order = nullptr, bool ranked = false)
+                               const int32_t* order = nullptr, bool ranked = false, bool rankInline = false)
 {
     if (numActive == 0) return hipSuccess;
     hipError_t err = hipSuccess;
     int vec = pick_vec(g, y, transpose ? nullptr : x);
     const int vsrc = pick_vec(g, ysrc, nullptr);
     if (vsrc < vec) vec = vsrc;
-    if (vec == 4) scatter_mode<4>(x, y, ysrc, idx, g, numActive, transpose, mode, stream, err, order, ranked);
-    else if (vec == 2) scatter_mode<2>(x, y, ysrc, idx, g, numActive, transpose, mode, stream, err, order, ranked);
-    else scatter_mode<1>(x, y, ysrc, idx, g, numActive, transpose, mode, stream, err, order, ranked);
+    if (vec == 4) scatter_mode<4>(x, y, ysrc, idx, g, numActive, transpose, mode, stream, err, order, ranked, rankInline);
+    else if (vec == 2) scatter_mode<2>(x, y, ysrc, idx, g, numActive, transpose, mode, stream, err, order, ranked, rankInline);
+    else scatter_mode<1>(x, y, ysrc, idx, g, numActive, transpose, mode, stream, err, order, ranked, rankInline);
     if (err != hipSuccess) return err;
     return hipGetLastError();
 }
@@ -999,11 +1045,30 @@ static bool build_owner_map(const int16_t* idx, int numActive, const Geom& g, vo
     return true;
 }
 
+// The planar tile kernel can rank the blocks itself (SCATTER_RANKED_INLINE): planar stack, at most 2x2 blocks over
+// a pixel, a list short enough that a workgroup's share of the comparison stays small against its tile.
+constexpr int RANK_INLINE_MAX_BLOCKS = 2048;
+
+static bool rank_inline_applies(const Geom& g, int numActive, bool transpose, int vec)
+{
+    if (!transpose || numActive > RANK_INLINE_MAX_BLOCKS || !(g.U < g.R || g.V < g.S)) return false;
+    if (g.R > 2 * (int64_t)g.U || g.S > 2 * (int64_t)g.V || (int64_t)g.R * g.S < 4) return false;
+    TileArgs a;
+    int threads;
+    size_t lds;
+    unsigned grid;
+    return scatter_tile_args(g, numActive, vec, a, threads, lds, grid);  // else k_planar_small would run
+}
+
 hipError_t launch_scatter_owned(const float* x, float* y, const int16_t* idx, int numActive, const Geom& g,
                                 bool transpose, void* workspace, size_t workspaceBytes, hipStream_t stream, bool& done)
 {
     done = false;
     if (numActive == 0) { done = true; return hipSuccess; }
+    if (rank_inline_applies(g, numActive, transpose, pick_vec(g, y, nullptr))) {
+        done = true;
+        return scatter_from(x, y, y, idx, numActive, g, transpose, SCATTER_ASSIGN, stream, nullptr, false, true);
+    }
     if (rank_table_applies(g, numActive) && scatter_owner_workspace_bytes(g, numActive) != 0 && workspace &&
         workspaceBytes >= (size_t)numActive * 4 + 16 && (reinterpret_cast<uintptr_t>(workspace) & 3) == 0) {
         int32_t* table = static_cast<int32_t*>(workspace);
