@@ -22,8 +22,17 @@ holds per-op device times (HIP events around batches of back-to-back launches on
 `--density`, `ops_by_density` the same at 5 %, 15 % and 30 %,
 `roofline` the dominant kernel (the slower of gather and scatter) against the 8 TB/s HBM peak, `cpu_baseline`
 the single-threaded CPU oracle (the reference's CPU functors restated; the reference builds them
-without OpenMP) on the same workload on this machine's host cores.  Tables for the other
-configurations (`--all-configs`) go to stderr.
+without OpenMP) on the same workload on this machine's host cores.  `ops_nhwc` times the same gather and
+scatter with transpose=False (the reference's default layout), `configs` holds the other four benchmark
+configurations (end to end and per op), `reference_layer_sizes` the three shapes on which the reference's own
+test times gather + scatter (sbnet_ops/tests/test_sparse_blocks.py:440-443).
+
+Every per-op entry carries two byte counts.  `algorithmic_bytes` is the reference's data flow (the table below).
+`moved_bytes` is what this implementation has to move for the same result: an ordered overlapping write stores
+every covered pixel once, not once per covering block; the owner-computes overlapping add reads and writes every
+covered pixel once and reads only the in-image part of the stack; the copying scatter is built in one pass (the
+base is read where it is needed and the output written once) instead of copy-then-scatter.  Fractions of the
+8 TB/s peak are given for both; the second is the one that says how close the kernel is to the memory system.
 
 Algorithmic bytes (B = bsize[0]*bsize[1]*C*4 per block, B_in its in-image part, M active blocks):
   gather            M*(B_in + B) + 6*M      read x once per block element, write the stack
@@ -83,6 +92,16 @@ def in_image_bytes(idx, bsize, bstride, boffset, H, W, C):
     return int((rows * cols).sum()) * C * 4
 
 
+def covered_pixels(idx, bsize, bstride, boffset, N, H, W):
+    """Number of distinct in-image pixels that the blocks of the list cover."""
+    cov = np.zeros((N, H, W), bool)
+    for n, bh, bw in np.asarray(idx, np.int64):
+        if 0 <= n < N:
+            h0, w0 = boffset[0] + bh * bstride[0], boffset[1] + bw * bstride[1]
+            cov[n, max(h0, 0):max(h0 + bsize[0], 0), max(w0, 0):max(w0 + bsize[1], 0)] = True
+    return int(cov.sum())
+
+
 class Path:
     """Pre-allocated device buffers and raw C-ABI calls for one workload, `nsets` rotating copies."""
 
@@ -129,8 +148,11 @@ class Path:
                 s["mask"] = None
                 s["idx"] = torch.from_numpy(idx_host).to(dev)
             s["ws"] = torch.empty(max(self.nws, 16), dtype=torch.uint8, device=dev)
-            nsw = lib.sbnet_sparse_scatter_workspace_bytes(self.M, self.dims, 4, self.sbs, 2, self.sbst, 2, self.sbo, 2) \
-                if ((wl.s_add and wl.s_atomic and not wl.transpose) or not wl.s_var) else 0
+            # every scatter is given the scratch the library asks for: overlapping adds then run without atomics,
+            # overlapping plain writes land in the CPU functor's order, the copying op is built in one pass
+            # (sized for the whole list, which the device-count entry points take as their capacity)
+            nsw = lib.sbnet_sparse_scatter_workspace_bytes(max(self.M, self.maxidx), self.dims, 4, self.sbs, 2, self.sbst,
+                                                           2, self.sbo, 2)
             s["sws"] = torch.empty(nsw, dtype=torch.uint8, device=dev) if nsw else None
             s["dcount"] = torch.zeros(1, dtype=torch.int32, device=dev)
             if wl.x is not None:
@@ -156,11 +178,23 @@ class Path:
         bin_g = in_image_bytes(idx_host, wl.bsize, wl.bstride, wl.boffset, H, W, C)
         bin_s = in_image_bytes(idx_host, wl.s_bsize, wl.s_bstride, wl.s_boffset, H, W, C)
         M = self.M
+        full = N * H * W * C * 4
         self.bytes = {
             "reduce_mask": N * H * W * 4 + 6 * M + 4,
             "gather": bin_g + M * B + 6 * M,
-            "scatter": M * sB + (2 if wl.s_add else 1) * bin_s + 6 * M + (0 if wl.s_var else 2 * N * H * W * C * 4),
+            "scatter": M * sB + (2 if wl.s_add else 1) * bin_s + 6 * M + (0 if wl.s_var else 2 * full),
         }
+        # what this implementation has to move (see the module docstring)
+        cov = covered_pixels(idx_host, wl.s_bsize, wl.s_bstride, wl.s_boffset, N, H, W) * C * 4
+        if not wl.s_var:
+            sc = M * sB + (full if wl.s_add else full - cov) + full + 6 * M
+        elif not wl.s_add:
+            sc = M * sB + cov + 6 * M
+        elif wl.s_atomic:
+            sc = bin_s + 2 * cov + 6 * M
+        else:
+            sc = M * sB + 2 * bin_s + 6 * M
+        self.moved = {"reduce_mask": self.bytes["reduce_mask"], "gather": self.bytes["gather"], "scatter": sc}
 
     def check(self, rc):
         if rc != 0:
@@ -208,10 +242,11 @@ class Path:
         self.check(self.lib.sbnet_sparse_gather_device_count(
             s["x"].data_ptr(), self.dims, 4, s["dcount"].data_ptr(), self.maxidx, s["idx"].data_ptr(), self.bs, 2,
             self.bst, 2, self.bo, 2, int(wl.transpose), s["stack_cap"].data_ptr(), self.stream))
+        ws = s["sws"]
         self.check(self.lib.sbnet_sparse_scatter_var_device_count(
             s["stack_cap"].data_ptr(), s["dcount"].data_ptr(), self.maxidx, s["idx"].data_ptr(), s["base"].data_ptr(),
             self.dims, 4, self.sbs, 2, self.sbst, 2, self.sbo, 2, int(wl.s_add), int(wl.s_atomic), int(wl.transpose),
-            None, 0, self.stream))
+            ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0, self.stream))
 
     def step(self, i):
         M = self.reduce(i) if self.wl.mask is not None else self.M
@@ -250,30 +285,20 @@ class Path:
         if self.wl.x is not None:
             ops["gather"] = self.time_op(lambda i: self.gather(i, self.M))
         ops["scatter"] = self.time_op(lambda i: self.scatter(i, self.M))
-        wl = self.wl
-        if wl.s_var and not wl.s_add and (wl.s_bstride[0] < wl.s_bsize[0] or wl.s_bstride[1] < wl.s_bsize[1]):
-            # the same scatter given scratch: overlapping plain writes in the CPU functor's order (owner map built
-            # by two small launches, then the scatter with one owner read per pixel)
-            nsw = self.lib.sbnet_sparse_scatter_workspace_bytes(self.M, self.dims, 4, self.sbs, 2, self.sbst, 2,
-                                                                self.sbo, 2)
-            for s in self.sets:
-                s["sws"] = self.torch.empty(nsw, dtype=self.torch.uint8, device="cuda:0")
-            ops["scatter_ordered"] = self.time_op(lambda i: self.scatter(i, self.M))
-            self.bytes["scatter_ordered"] = self.bytes["scatter"]
-            for s in self.sets:
-                s["sws"] = None
         table = {}
         for k, us in ops.items():
-            gbs = self.bytes[k] / us * 1e-3
-            table[k] = {"us": round(us, 2), "bytes": self.bytes[k], "GBps": round(gbs, 1),
-                        "frac_of_8TBps": round(gbs / HBM_PEAK_GBS, 4)}
+            gbs, mgbs = self.bytes[k] / us * 1e-3, self.moved[k] / us * 1e-3
+            table[k] = {"us": round(us, 2), "algorithmic_bytes": self.bytes[k], "moved_bytes": self.moved[k],
+                        "GBps": round(gbs, 1), "frac_of_8TBps": round(gbs / HBM_PEAK_GBS, 4),
+                        "moved_GBps": round(mgbs, 1), "moved_frac_of_8TBps": round(mgbs / HBM_PEAK_GBS, 4)}
         return table
 
 
 class BenchSet(ctypes.Structure):   # struct sbnet_bench_set of sbnet_amd/csrc/sbnet_bench_loop.cpp
     _fields_ = [("mask", ctypes.c_void_p), ("x", ctypes.c_void_p), ("base", ctypes.c_void_p),
                 ("stack", ctypes.c_void_p), ("idx", ctypes.c_void_p), ("count_dev", ctypes.c_void_p),
-                ("reduce_ws", ctypes.c_void_p), ("reduce_ws_bytes", ctypes.c_size_t)]
+                ("reduce_ws", ctypes.c_void_p), ("reduce_ws_bytes", ctypes.c_size_t),
+                ("scatter_ws", ctypes.c_void_p), ("scatter_ws_bytes", ctypes.c_size_t)]
 
 
 class BenchGeom(ctypes.Structure):  # struct sbnet_bench_geom
@@ -305,8 +330,10 @@ def cxx_pipeline(path, steps, warmup, batches):
                         dtype=torch.float32, device="cuda:0") for _ in path.sets]
     sets = (BenchSet * len(path.sets))()
     for k, s in enumerate(path.sets):
+        sws = s["sws"]
         sets[k] = BenchSet(s["mask"].data_ptr(), s["x"].data_ptr(), s["base"].data_ptr(), caps[k].data_ptr(),
-                           s["idx"].data_ptr(), s["dcount"].data_ptr(), s["ws"].data_ptr(), path.nws)
+                           s["idx"].data_ptr(), s["dcount"].data_ptr(), s["ws"].data_ptr(), path.nws,
+                           sws.data_ptr() if sws is not None else None, sws.numel() if sws is not None else 0)
     g = BenchGeom(path.N, path.H, path.W, path.C, I2(*wl.bcount), I2(*wl.bsize), I2(*wl.bstride), I2(*wl.boffset),
                   I2(*wl.s_bsize), I2(*wl.s_bstride), I2(*wl.s_boffset), wl.tol, int(wl.avgpool), int(wl.transpose),
                   int(wl.s_add), int(wl.s_atomic), path.maxidx)
@@ -554,7 +581,7 @@ def main():
     roofline = {"bound": "hbm", "kernel": kernel_names[dom],
                 "achieved": g["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(g["GBps"] / HBM_PEAK_GBS, 4), "us_per_launch": g["us"],
-                "algorithmic_bytes_per_launch": g["bytes"],
+                "algorithmic_bytes_per_launch": g["algorithmic_bytes"], "moved_bytes_per_launch": g["moved_bytes"],
                 "traffic": traffic, "traffic_source": traffic_note}
     if traffic:
         # the same launch time against the bytes the profiler counted between L2 and the fabric
@@ -595,14 +622,43 @@ def main():
         out["cpu_baseline_openmp"] = omp
         gpu_gs = nb / ((ops["gather"]["us"] + ops["scatter"]["us"]) * 1e-6) * 1e-9
         out["gather_plus_scatter_GBps"] = round(gpu_gs, 1)
+    del path
+    torch.cuda.empty_cache()
+
+    # the same two ops in the reference's default layout (transpose=False), same workload
+    p = Path(workloads.config3(args.density)._replace(transpose=False), torch, lib, nsets=3)
+    t = p.op_table()
+    out["ops_nhwc"] = {"gather": t["gather"], "scatter": t["scatter"], "M": p.M,
+                       "note": "sparse_gather / sparse_scatter_var with transpose=False (NHWC block stack), %s" % p.wl.name}
+    del p
+    torch.cuda.empty_cache()
+
+    # the other benchmark configurations, each end to end (host-visible count) and per op
+    out["configs"] = {name: config_row(name, torch, lib, workloads) for name in ("C1", "C2", "C4", "C5")}
+
+    # the shapes the reference's own test times its gather + scatter on (timed region: both ops)
+    layers = {}
+    for size in workloads.REFERENCE_LAYER_SIZES:
+        for transpose in (False, True):
+            p = Path(workloads.reference_layer(size, transpose), torch, lib, nsets=3)
+            t = p.op_table()
+            layers["%dx%dx%d %s" % (size + ("transpose" if transpose else "nhwc",))] = {
+                "M": p.M, "gather": t["gather"], "scatter": t["scatter"],
+                "gather_plus_scatter_us": round(t["gather"]["us"] + t["scatter"]["us"], 2)}
+            del p
+            torch.cuda.empty_cache()
+    out["reference_layer_sizes"] = {
+        "note": "benchmarkLayerSizes of the reference's test (18x18 blocks at stride 18, offset (-1,-2), every block "
+                "active): sparse_gather, then the copying sparse_scatter(add=False); the reference times both ops "
+                "together with its in-graph timers",
+        "rows": layers}
     print(json.dumps(out))
     sys.stdout.flush()
 
     if args.all_configs:
-        del path
-        torch.cuda.empty_cache()
         for name in CONFIGS:
-            print(json.dumps(config_row(name, torch, lib, workloads)), file=sys.stderr)
+            if name.startswith("C3"):
+                print(json.dumps(config_row(name, torch, lib, workloads)), file=sys.stderr)
 
 
 CONFIGS = ["C1", "C2", "C3@5%", "C3@15%", "C3@30%", "C4", "C5"]
@@ -625,7 +681,13 @@ def config_row(name, torch, lib, workloads):
         p.step(i % n)
     torch.cuda.synchronize()
     e2e = (time.perf_counter() - t0) / K * 1e6
-    row = {"config": name, "M": p.M, "end_to_end_us": round(e2e, 1), "ops": p.op_table()}
+    wl = p.wl
+    row = {"config": name, "M": p.M, "end_to_end_us": round(e2e, 1), "ops": p.op_table(),
+           "workload": "x=%s bsize %s bstride %s boffset %s %s-pool tol %g; gather transpose=%s; %s add=%s atomic=%s "
+                       "bsize %s bstride %s boffset %s" % (
+                           wl.shape, wl.bsize, wl.bstride, wl.boffset, "avg" if wl.avgpool else "max", wl.tol,
+                           wl.transpose, "sparse_scatter_var" if wl.s_var else "sparse_scatter", wl.s_add, wl.s_atomic,
+                           wl.s_bsize, wl.s_bstride, wl.s_boffset)}
     del p
     torch.cuda.empty_cache()
     return row

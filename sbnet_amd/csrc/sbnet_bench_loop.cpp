@@ -20,6 +20,8 @@ struct sbnet_bench_set {
     int32_t* count_dev;         // [1]
     void* reduce_ws;
     size_t reduce_ws_bytes;
+    void* scatter_ws;           // scratch of sbnet_sparse_scatter_workspace_bytes() for max_active blocks, or NULL
+    size_t scatter_ws_bytes;
 };
 
 struct sbnet_bench_geom {
@@ -61,7 +63,8 @@ int sbnet_bench_pipeline(const sbnet_bench_set* sets, int nsets, const sbnet_ben
                                      g->transpose, b.stack, stream);
             if (rc) return rc;
             rc = sbnet_sparse_scatter_var(b.stack, count, b.idx, b.base, dims, 4, g->s_bsize, 2, g->s_bstride, 2,
-                                          g->s_boffset, 2, g->add, g->atomic, g->transpose, nullptr, 0, stream);
+                                          g->s_boffset, 2, g->add, g->atomic, g->transpose, b.scatter_ws,
+                                          b.scatter_ws_bytes, stream);
             if (rc) return rc;
         } else {
             rc = sbnet_reduce_mask(b.mask, g->N, g->H, g->W, g->bcount, 2, g->bsize, 2, g->bstride, 2, g->boffset, 2,
@@ -73,7 +76,8 @@ int sbnet_bench_pipeline(const sbnet_bench_set* sets, int nsets, const sbnet_ben
             if (rc) return rc;
             rc = sbnet_sparse_scatter_var_device_count(b.stack, b.count_dev, g->max_active, b.idx, b.base, dims, 4,
                                                        g->s_bsize, 2, g->s_bstride, 2, g->s_boffset, 2, g->add,
-                                                       g->atomic, g->transpose, nullptr, 0, stream);
+                                                       g->atomic, g->transpose, b.scatter_ws, b.scatter_ws_bytes,
+                                                       stream);
             if (rc) return rc;
         }
     }

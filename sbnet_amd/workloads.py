@@ -157,6 +157,28 @@ def config5(seed=1005, with_x=True):
                s_add=True, s_atomic=False, s_var=False, x=x, mask=mask)
 
 
+REFERENCE_LAYER_SIZES = [(300, 480, 64), (600, 960, 64), (300, 480, 256)]
+
+
+def reference_layer(size, transpose=True, seed=1006, with_x=True):
+    """The shapes on which the reference's own test times gather + scatter (benchmarkLayerSizes,
+    sbnet_ops/tests/test_sparse_blocks.py:440-443, through runTestForOneSize :139-260 and generateInputs :124-133):
+    one image [1,H,W,C], mask and x ~ N(0,1), 18x18 blocks at stride 18, offset (-1,-2), block counts by that
+    file's covering rule (:101-121), max pooling with tol = the 70th percentile of x (which leaves every block
+    active: some pixel of 324 exceeds it), gather, then the copying scatter with add=False and the same geometry."""
+    H, W, C = size
+    rng = np.random.default_rng(seed + H + C)
+    mask = rng.standard_normal((1, H, W, 1), dtype=np.float32)
+    x = rng.standard_normal((1, H, W, C), dtype=np.float32) if with_x else None
+    sample = x if x is not None else rng.standard_normal(1 << 20, dtype=np.float32)
+    tol = float(np.percentile(sample.reshape(-1)[:1 << 22], 70))
+    bsize, bstride, boffset = [18, 18], [18, 18], [-1, -2]
+    bcount = [1 + (H - boffset[0] - 1) // bstride[0], 1 + (W - boffset[1] - 1) // bstride[1]]
+    return _wl(name="L%dx%dx%d" % size, shape=[1, H, W, C], bsize=bsize, bstride=bstride, boffset=boffset, bcount=bcount,
+               tol=tol, avgpool=False, transpose=transpose, s_bsize=bsize, s_bstride=bstride, s_boffset=boffset,
+               s_add=False, s_atomic=False, s_var=False, x=x, mask=mask)
+
+
 def centre_crop(stack, bsize, s_bsize, transpose):
     """Stand-in for the VALID convolution between gather and scatter: keeps the centre s_bsize window of
     every gathered block (numpy or torch)."""

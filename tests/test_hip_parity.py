@@ -1135,7 +1135,7 @@ def test_functor_level_entry_points():
 # the five benchmark configurations at full size
 # ---------------------------------------------------------------------------------------------
 
-def run_workload(wl):
+def run_workload(wl, base=None):
     """reduce_mask -> gather -> (centre crop) -> scatter on a Workload, compared op by op."""
     idx_o, cnt_o, r = check_reduce(wl.mask, wl.bcount, wl.bsize, wl.bstride, wl.boffset, wl.tol, wl.avgpool)
     M = int(cnt_o[0])
@@ -1146,7 +1146,8 @@ def run_workload(wl):
     np.testing.assert_array_equal(host(g), g_o)
     q = workloads.centre_crop(g, wl.bsize, wl.s_bsize, wl.transpose).contiguous()
     q_o = np.ascontiguousarray(workloads.centre_crop(g_o, wl.bsize, wl.s_bsize, wl.transpose))
-    base = np.zeros(wl.shape, np.float32) if wl.name == "C1" else wl.x
+    if base is None:
+        base = np.zeros(wl.shape, np.float32) if wl.name == "C1" else wl.x
     fn = sbnet_amd.sparse_scatter_var if wl.s_var else sbnet_amd.sparse_scatter
     bd = dev(base)
     y = fn(q, r.bin_counts, r.active_block_indices, bd, wl.s_bsize, wl.s_bstride, wl.s_boffset, add=wl.s_add,
@@ -1163,6 +1164,17 @@ def run_workload(wl):
                             wl.s_add, wl.s_atomic, wl.transpose, use_var=True, scratch=False)
         np.testing.assert_array_equal(host(bd2), y_o)
     return M
+
+
+@pytest.mark.parametrize("transpose", [False, True])
+@pytest.mark.parametrize("size", workloads.REFERENCE_LAYER_SIZES, ids=str)
+def test_reference_layer_sizes(size, transpose):
+    """The three shapes the reference's test times its ops on (benchmarkLayerSizes, test_sparse_blocks.py:440-443):
+    18x18 blocks at stride 18, offset (-1,-2), every block active, copying scatter onto a base of 10.0
+    (test_sparse_blocks.py:161, 228), full size, op by op against the oracle."""
+    wl = workloads.reference_layer(size, transpose)
+    M = run_workload(wl, base=np.full(wl.shape, 10.0, np.float32))
+    assert M == wl.bcount[0] * wl.bcount[1]
 
 
 def test_config1_plumbing():
