@@ -206,21 +206,34 @@ size_t sbnet_sparse_scatter_workspace_bytes(int32_t num_active, const int64_t* y
  *   add=1, atomic=0 requires bstride >= bsize on both axes (sparse_gather.cc:322-326).
  *   add=0 with overlapping blocks (bstride < bsize): the reference's CPU functor walks the list front to
  *   back, so the block listed last wins on a pixel that several blocks cover (sparse_gather.cc:105-129).
- *   Given scratch (below) this library writes exactly that, for both stack layouts and for lists that name
- *   a block twice.  Without scratch, as in the reference's GPU path, which block wins is unspecified unless
- *   the overlapping values are equal.
+ *   This library writes exactly that, for both stack layouts and for lists that name a block twice: without
+ *   scratch when the stack is planar (transpose=1), at most 2x2 blocks cover a pixel (bsize <= 2*bstride) and
+ *   the list has at most 2048 blocks (the kernel that moves a block compares it with the rows listed after
+ *   it); otherwise given scratch (below).  Where neither holds, as in the reference's GPU path, which block
+ *   wins is unspecified unless the overlapping values are equal.
  *   workspace   optional device scratch (4-byte aligned) of sbnet_sparse_scatter_workspace_bytes() bytes,
  *               or NULL.  Three uses.
- *               (0) add=0 and bstride < bsize: every block writes only the pixels that no block listed later
- *               covers: the CPU functor's result, no pixel written twice.  Which pixels those are comes from one
- *               small extra launch that compares the blocks of the list pairwise (at most 2x2 blocks over a
- *               pixel, bsize <= 2*bstride, and at most 4096 blocks; in-place op), or else from an owner map (one
- *               int32 per pixel: the last listed block that covers it) built by two extra launches.
- *               (1) sbnet_sparse_scatter with atomic=0: when the blocks cover 16 MB or more, y is built from
- *               two disjoint parts instead of "copy ybase, scatter on top": pixels that no active block covers
- *               are copied from ybase, covered ones are written by the scatter, which reads ybase where it
- *               adds.  Same y, every byte moved once (one flag byte per pixel in the scratch tells the parts
- *               apart).
+ *               (0) add=0 and bstride < bsize, where the kernel cannot order the blocks itself (NHWC stack,
+ *               long lists, more than 2x2 blocks over a pixel): every block writes only the pixels that no
+ *               block listed later covers: the CPU functor's result, no pixel written twice.  Which pixels
+ *               those are comes from one small extra launch that compares the blocks of the list pairwise (at
+ *               most 2x2 blocks over a pixel and at most 4096 blocks; in-place op), or else from an owner map
+ *               (one int32 per pixel: the last listed block that covers it) built by two extra launches.
+ *               (1) sbnet_sparse_scatter with atomic=0 and blocks that do not overlap (bstride >= bsize): y is
+ *               built in one pass over its bytes instead of "copy ybase, scatter on top".  Two small launches
+ *               put an inverse map (block position -> list position) into the scratch; one streaming kernel
+ *               then walks y in row order, reads ybase where the result needs it (all of it for an add, the
+ *               uncovered pixels for a plain write), reads the block stack where a block covers the pixel and
+ *               writes y once.  Same y, every byte moved once.  A list that names a block several times gets
+ *               the CPU functor's result here as well (the last of the rows wins a plain write, an add sums
+ *               all of them in list order).  A planar stack (transpose=1) is staged through LDS by the same
+ *               kernel when bsize[1] and bstride[1] are multiples of 4, bstride[1] divides the kernel's strip
+ *               width (256 channel vectors, i.e. 32 pixels at 32 channels or more) and boffset[1] is a
+ *               multiple of bstride[1]; other planar geometries take two passes once the blocks cover 16 MB
+ *               (copy of the uncovered pixels, then the scatter kernel, which reads ybase where it adds), and
+ *               copy-then-scatter below that: in these two cases rows that name the same block race as they
+ *               do in the reference's GPU kernels.  Overlapping plain writes (add=0, bstride < bsize) from
+ *               16 MB of blocks on use the owner map of (0) as their coverage record in the same way.
  *               (2) add=1, atomic=1: with it the overlapping adds need no atomics:
  *               - transpose=0 and at most 2x2 blocks per pixel: each pixel is summed by one owner in ascending
  *                 block-list order, bit-identical to the reference's sequential CPU functor;

@@ -26,8 +26,8 @@ struct Geom {
 
 enum ScatterMode { SCATTER_ASSIGN = 0, SCATTER_ADD = 1, SCATTER_ATOMIC = 2 };
 
-// reduce_mask scratch: words of the one-launch mode, one flag byte per sparsity block, one int32 count per
-// pooling workgroup, one int32 for the total when the caller gives no device count.  Its contents before a
+// reduce_mask scratch: one flag byte per sparsity block, one int32 count per pooling workgroup, one int32 for
+// the total when the caller gives no device count.  Its contents before a
 // call do not matter.  reduce_mask_count_slot: where the total goes when the caller gives no device count.
 size_t reduce_mask_workspace_bytes(int64_t totalBlocks);
 int32_t* reduce_mask_count_slot(void* workspace, int64_t totalBlocks);
@@ -77,11 +77,15 @@ size_t scatter_owner_workspace_bytes(const Geom& g, int numActive);
 hipError_t launch_scatter_owned(const float* x, float* y, const int16_t* idx, int numActive, const Geom& g,
                                 bool transpose, void* workspace, size_t workspaceBytes, hipStream_t stream, bool& done);
 
-// y = copy of ybase with the blocks written ("=") or added ("+=", non-overlapping) on top, moving every byte once:
-// pixels that no active block covers are copied, covered ones are written by the scatter kernels, which read
-// ybase where they add.  Needs scratch of scatter_cover_workspace_bytes() for one flag byte per pixel; `done` is
-// false when the method does not apply (no scratch, atomic mode, too little coverage to pay for preparing the
-// flags) and nothing was launched: the caller then copies ybase and scatters in place.
+// y = copy of ybase with the blocks written ("=") or added ("+=", non-overlapping) on top, moving every byte once.
+// Blocks that do not overlap: an inverse map (cell of the block grid -> list position) in the scratch, then one
+// streaming kernel over y that reads ybase where the result needs it, the stack where a block covers the pixel,
+// and writes y once (planar stacks of geometries the kernel does not stage: a pass that copies the uncovered
+// pixels, then the scatter kernels, which read ybase where they add).  Overlapping plain writes: the owner map of
+// the ordered scatter as coverage record, a copy of the uncovered pixels, then the ordered scatter.  Needs scratch
+// of scatter_cover_workspace_bytes() / scatter_owner_workspace_bytes(); `done` is false when the method does not
+// apply (no scratch, atomic mode, too little coverage to pay for the extra launches) and nothing was launched:
+// the caller then copies ybase and scatters in place.
 size_t scatter_cover_workspace_bytes(const Geom& g, int numActive);
 hipError_t launch_scatter_over_base(const float* x, const float* ybase, float* y, const int16_t* idx, int numActive,
                                     const Geom& g, bool transpose, ScatterMode mode, void* workspace,

@@ -864,14 +864,292 @@ hipError_t launch_scatter_colored(const float* x, float* y, const int16_t* idx, 
     return hipGetLastError();
 }
 
-// ---- "copy of the base + scatter" without copying what the scatter overwrites -------------------
+// ---- "copy of the base + scatter" in one pass -------------------------------------------------------
 //
 // sparse_scatter (not the in-place op) returns a fresh tensor: the base, with the blocks written or added on
-// top (sparse_gather.cc:338-346 copies the whole base, then scatters).  Copy-then-scatter moves every
-// covered pixel twice more than needed.  With one flag byte per pixel ("an active block covers it") the work
-// splits into two disjoint parts: k_copy_uncovered copies the pixels without the flag, and the ordinary
-// scatter kernels write the flagged ones, reading the base (`ysrc`) where they add.  Same result, every byte
-// moved once.  The flags cost N*H*W bytes of scratch and two small launches (clear, mark).
+// top (sparse_gather.cc:338-346 copies the whole base, then scatters).  Copy-then-scatter moves every covered
+// pixel twice more than needed.
+//
+// Blocks that do not overlap (bstride >= bsize on both axes, which add without atomics requires anyway,
+// sparse_gather.cc:322-326): the plane divides into cells of bstride[0] x bstride[1] pixels, cell (bh, bw)
+// holds block (bh, bw) in its first bsize rows and columns, and a pixel can only be written by the block of its
+// own cell.  With an inverse map "cell -> list position" (k_pull_fill, k_cell_map) ONE streaming kernel
+// (k_scatter_strip) walks the output in row order: a workgroup takes a strip of 4 image rows of one row of
+// cells, 256 channel vectors wide; a lane looks its cell up once, reads the base where the result needs it (all
+// of it for an add, the uncovered pixels for a plain write), reads the block stack where a block covers the
+// pixel, and writes the output once.  No flag bytes, no second pass over the covered pixels.
+//
+// Overlapping plain writes keep the owner map of the ordered scatter as their coverage record (k_copy_uncovered,
+// then the ordinary scatter kernels, which read the base where they add).
+
+struct StripArgs {
+    Geom g;
+    int bhMin, bwMin, nBH, nBW;  // cells that touch the image: bh in [bhMin, bhMin + nBH), likewise bw
+    uint32_t kPerBand;           // strips per row of cells: ceil(U / STRIP_ROWS)
+    uint32_t CV;                 // channel vectors per pixel
+    uint32_t CVT;                // channel vectors per pixel that one strip moves (a chunk of the channels)
+    uint32_t CT;                 // the same in floats
+    uint32_t nCC;                // channel chunks: ceil(CV / CVT)
+    uint32_t PX;                 // pixels per strip: 256 / CVT
+    uint32_t imgBytes;
+    int64_t imgFloats;
+    uint32_t swzMask;            // LDS staging of a planar stack: see strip_lds_index
+    uint32_t nPC;                // pixel chunks per image row: ceil(W / PX)
+    uint32_t tiles;              // strips in all: N * nBH * kPerBand * nPC * nCC
+    uint32_t S4;                 // planar stack: 16-byte slots per block row, S / 4
+    uint32_t cellsPerStrip;      // planar stack: PX / V
+    FastDiv dCVT, dV, dK, dCC, dPC, dBH, dS4, dCT;
+};
+
+constexpr int STRIP_ROWS = 4;
+
+// Cell of block (n, bh, bw) in the map, or -1 when the block cannot touch the image.
+__device__ __forceinline__ int64_t cell_slot(const StripArgs& a, int n, int bh, int bw)
+{
+    if ((unsigned)n >= (unsigned)a.g.N) return -1;
+    const int ih = bh - a.bhMin, iw = bw - a.bwMin;
+    if ((unsigned)ih >= (unsigned)a.nBH || (unsigned)iw >= (unsigned)a.nBW) return -1;
+    return ((int64_t)n * a.nBH + ih) * a.nBW + iw;
+}
+
+// One thread per list row: the row's position goes into its cell.  A cell named by several rows keeps them as a
+// linked list (the map holds the row that arrived last, chain[row] the one it displaced) and raises `dup`; the
+// main kernel then walks the lists, so that a plain write still takes the row listed last and an add still sums
+// in list order, as the sequential CPU functor does (sparse_gather.cc:105-129).
+__global__ __launch_bounds__(256) void k_cell_map(const int16_t* __restrict__ idx, int numActive, StripArgs a,
+                                                   int32_t* __restrict__ map, int32_t* __restrict__ chain,
+                                                   int32_t* __restrict__ dup)
+{
+    const int ib = (int)(blockIdx.x * 256 + threadIdx.x);
+    if (ib >= numActive || (a.g.countDev && ib >= *a.g.countDev)) return;
+    const int64_t slot = cell_slot(a, idx[(size_t)ib * 3], idx[(size_t)ib * 3 + 1], idx[(size_t)ib * 3 + 2]);
+    int32_t prev = -1;
+    if (slot >= 0) {
+        prev = atomicExch(map + slot, ib);
+        if (prev >= 0) *dup = 1;
+    }
+    chain[ib] = prev;
+}
+
+// VEC channels of block ib at block pixel (r, s), channel vector cv.
+template <int VEC, bool PLANAR>
+__device__ __forceinline__ typename Vec<VEC>::type strip_stack_load(const float* __restrict__ x, int ib, int r,
+                                                                    uint32_t s, uint32_t cv, const StripArgs& a)
+{
+    typedef typename Vec<VEC>::type vec;
+    if (!PLANAR) {
+        const int64_t e = (((int64_t)ib * a.g.R + r) * a.g.S + s) * a.CV + cv;
+        return ld_stream(reinterpret_cast<const vec*>(x) + e);
+    }
+    vec v = vzero<VEC>();
+    const int64_t plane = (int64_t)a.g.R * a.g.S;
+    const float* __restrict__ p = x + ((int64_t)ib * a.g.C + cv * VEC) * plane + (int64_t)r * a.g.S + s;
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) vset(v, k, ld_stream(p + k * plane));
+    return v;
+}
+
+// Planar stack [blocks, C, R, S]: the strip's part of it goes through LDS, for geometries in which the strips line
+// up with the cells and the planar rows with 16-byte vectors (bsize[1], bstride[1] multiples of 4, bstride[1]
+// dividing the strip's width, boffset[1] a multiple of bstride[1]: the usual output geometry of a convolution over
+// the gathered blocks).  LDS holds the strip as [row][pixel][channel of the chunk], the order in which the NHWC side
+// consumes it (one 16-byte read per lane).  The loading side deals 16-byte slots to the threads in the stack's own
+// memory order (4 pixels of a planar row, then the strip's rows of that channel, then the channels, then the
+// cells), so that a wave reads long contiguous pieces: a whole block when the plane is 4x4.  Channels are
+// XOR-swizzled in units of 4 by the pixel group's number, which spreads the transposing writes over the banks and
+// keeps every pixel's 4-channel vectors whole.
+__device__ __forceinline__ uint32_t strip_lds_index(const StripArgs& a, uint32_t u, uint32_t px, uint32_t c)
+{
+    return (u * a.PX + px) * a.CT + (c ^ (((px >> 2) & a.swzMask) << 2));  // c: channel inside the strip's chunk
+}
+
+constexpr int STRIP_SLOTS = 4;  // 16-byte slots per thread: 256 threads x 4 x 16 B = the strip's 16 KB
+
+__device__ __forceinline__ void strip_stage_planar(const float* __restrict__ x, const int32_t* __restrict__ mapRow,
+                                                   const StripArgs& a, float* lds, uint32_t pc, uint32_t c0, int r0,
+                                                   int hTop)
+{
+    const uint32_t C = (uint32_t)a.g.C, S = (uint32_t)a.g.S;
+    const int64_t plane = (int64_t)a.g.R * a.g.S;
+    const uint32_t iw0 = pc * a.cellsPerStrip;  // the strip's first cell
+    int ib[STRIP_SLOTS];
+    uint32_t cl[STRIP_SLOTS], uu[STRIP_SLOTS], px[STRIP_SLOTS], col[STRIP_SLOTS];
+    bool use[STRIP_SLOTS];
+#pragma unroll
+    for (int k = 0; k < STRIP_SLOTS; ++k) {
+        const uint32_t p = threadIdx.x + (uint32_t)k * 256u;
+        // p = ((cell * CT + cl) * 4 + u) * S4 + q
+        uint32_t t = fdiv(p, a.dS4);
+        const uint32_t q = p - t * a.S4;
+        uu[k] = t & 3u;
+        t >>= 2;
+        const uint32_t cell = fdiv(t, a.dCT);
+        cl[k] = t - cell * a.CT;
+        col[k] = 4u * q;
+        px[k] = cell * (uint32_t)a.g.V + col[k];
+        const int r = r0 + (int)uu[k];
+        use[k] = cell < a.cellsPerStrip && iw0 + cell < (uint32_t)a.nBW && c0 + cl[k] < C && r < a.g.R &&
+                 (unsigned)(hTop + (int)uu[k]) < (unsigned)a.g.H && pc * a.PX + px[k] < (uint32_t)a.g.W;
+        ib[k] = use[k] ? mapRow[iw0 + cell] : -1;
+    }
+    f4 val[STRIP_SLOTS];
+#pragma unroll
+    for (int k = 0; k < STRIP_SLOTS; ++k) {
+        if (ib[k] >= 0) {
+            const float* __restrict__ src = x + ((int64_t)ib[k] * C + c0 + cl[k]) * plane + (int64_t)(r0 + (int)uu[k]) * S + col[k];
+            val[k] = ld_stream(reinterpret_cast<const f4*>(src));
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < STRIP_SLOTS; ++k) {
+        if (ib[k] >= 0) {
+            // (a block's last columns may lie beyond the image: those pixels are not consumed)
+            const uint32_t at = strip_lds_index(a, uu[k], px[k], cl[k]);
+            lds[at] = val[k].x;
+            lds[at + a.CT] = val[k].y;
+            lds[at + 2u * a.CT] = val[k].z;
+            lds[at + 3u * a.CT] = val[k].w;
+        }
+    }
+}
+
+// sparse_gather.cc:103-130 on top of a copy of ybase (sparse_gather.cc:338-346), non-overlapping blocks.
+// OP: STRIP_ASSIGN / STRIP_ADD write the whole output; STRIP_COPY writes only the pixels that no block covers and
+// leaves the covered ones to a scatter kernel that follows (planar stacks whose geometry the staging above does
+// not take).
+constexpr int STRIP_ASSIGN = 0, STRIP_ADD = 1, STRIP_COPY = 2;
+
+template <int VEC, int OP, bool PLANAR>
+__global__ __launch_bounds__(256) void k_scatter_strip(const float* __restrict__ x, const float* __restrict__ ybase,
+                                                       float* __restrict__ y, const int32_t* __restrict__ map,
+                                                       const int32_t* __restrict__ chain,
+                                                       const int32_t* __restrict__ dup, StripArgs a)
+{
+    typedef typename Vec<VEC>::type vec;
+    typedef const int32_t __attribute__((address_space(4))) * const_i32_ptr;
+    constexpr bool ADD = OP == STRIP_ADD;
+    const uint32_t tid = threadIdx.x;
+    // Which strip: channel chunk, pixel chunk, strip of the row of cells, row of cells, image, the first fastest:
+    // neighbouring workgroups write neighbouring pieces of the same image rows.
+    uint32_t l = blockIdx.x;
+    uint32_t t = fdiv(l, a.dCC);
+    const uint32_t cc = (uint32_t)__builtin_amdgcn_readfirstlane((int)(l - t * a.nCC));
+    l = t; t = fdiv(l, a.dPC);
+    const uint32_t pc = (uint32_t)__builtin_amdgcn_readfirstlane((int)(l - t * a.nPC));
+    l = t; t = fdiv(l, a.dK);
+    const int r0 = __builtin_amdgcn_readfirstlane((int)(l - t * a.kPerBand)) * STRIP_ROWS;  // first block row of the strip
+    l = t; t = fdiv(l, a.dBH);
+    const uint32_t band = (uint32_t)__builtin_amdgcn_readfirstlane((int)(l - t * (uint32_t)a.nBH));
+    const uint32_t n = (uint32_t)__builtin_amdgcn_readfirstlane((int)t);
+    const int hTop = a.g.oh + ((int)band + a.bhMin) * a.g.U + r0;  // the strip's first image row
+
+    const uint32_t wl = fdiv(tid, a.dCVT), cvl = tid - wl * a.CVT;
+    const uint32_t cv = cc * a.CVT + cvl;
+    const uint32_t w = pc * a.PX + wl;
+    const bool live = wl < a.PX && w < (uint32_t)a.g.W && cv < a.CV;
+
+    // the lane's cell: one look-up for the strip's rows (they lie in one row of cells)
+    const int32_t* __restrict__ mapRow = map + ((int64_t)n * a.nBH + band) * a.nBW;
+    const uint32_t dw = w - (uint32_t)(a.g.ow + a.bwMin * a.g.V);  // >= 0 for every pixel of the image
+    const uint32_t iw = fdiv(dw, a.dV), s = dw - iw * (uint32_t)a.g.V;
+    int ib = -1;
+    if (live && s < (uint32_t)a.g.S && r0 < a.g.R) ib = mapRow[iw];
+
+    const rsrc_t br = make_rsrc(ybase + (int64_t)n * a.imgFloats, a.imgBytes);
+    const rsrc_t yr = make_rsrc(y + (int64_t)n * a.imgFloats, a.imgBytes);
+    uint32_t off[STRIP_ROWS];
+    bool inBlock[STRIP_ROWS];  // (the same for the whole workgroup)
+#pragma unroll
+    for (int u = 0; u < STRIP_ROWS; ++u) {
+        const int h = hTop + u;
+        const bool rowLive = r0 + u < a.g.U && (unsigned)h < (unsigned)a.g.H;
+        inBlock[u] = r0 + u < a.g.R;
+        off[u] = live && rowLive ? (((uint32_t)h * (uint32_t)a.g.W + w) * a.CV + cv) * (uint32_t)(VEC * 4) : BUF_OOB;
+    }
+    vec b[STRIP_ROWS], v[STRIP_ROWS];
+    if (ADD) {
+        // an add reads the base everywhere: these loads do not wait for the look-up
+#pragma unroll
+        for (int u = 0; u < STRIP_ROWS; ++u) b[u] = buf_load<VEC>(br, off[u]);
+    }
+    if (OP == STRIP_COPY) {
+        // covered pixels (whichever rows of the list cover them) belong to the scatter kernel that follows
+#pragma unroll
+        for (int u = 0; u < STRIP_ROWS; ++u) {
+            if (ib >= 0 && inBlock[u]) off[u] = BUF_OOB;
+            b[u] = buf_load<VEC>(br, off[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < STRIP_ROWS; ++u) buf_store<BUF_NT>(yr, off[u], b[u]);
+        return;
+    }
+    const bool dups = *(const_i32_ptr)(reinterpret_cast<uintptr_t>(dup)) != 0;
+    if (!dups) {
+        const bool cov = ib >= 0;
+        if (!ADD) {
+#pragma unroll
+            for (int u = 0; u < STRIP_ROWS; ++u) b[u] = buf_load<VEC>(br, cov && inBlock[u] ? BUF_OOB : off[u]);  // covered pixels are not read
+        }
+        if (PLANAR && r0 < a.g.R) {
+            extern __shared__ __attribute__((aligned(16))) float lds[];
+            strip_stage_planar(x, mapRow, a, lds, pc, cc * a.CT, r0, hTop);
+            lds_barrier();
+#pragma unroll
+            for (int u = 0; u < STRIP_ROWS; ++u) {
+                v[u] = vzero<VEC>();
+                if (cov && inBlock[u] && off[u] != BUF_OOB) {
+                    if (VEC == 4) {
+                        const f4 q = lds_read4(lds + strip_lds_index(a, (uint32_t)u, wl, cvl * 4u));
+#pragma unroll
+                        for (int k = 0; k < VEC; ++k) vset(v[u], k, vget(q, k));
+                    } else {
+#pragma unroll
+                        for (int k = 0; k < VEC; ++k) vset(v[u], k, lds[strip_lds_index(a, (uint32_t)u, wl, cvl * VEC + k)]);
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < STRIP_ROWS; ++u) {
+                v[u] = vzero<VEC>();
+                if (cov && inBlock[u] && off[u] != BUF_OOB) v[u] = strip_stack_load<VEC, false>(x, ib, r0 + u, s, cv, a);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < STRIP_ROWS; ++u) {
+            const bool hit = cov && inBlock[u];
+            buf_store<BUF_NT>(yr, off[u], hit ? (ADD ? vadd(b[u], v[u]) : v[u]) : b[u]);
+        }
+        return;
+    }
+    // Some cell is named by several rows of the list (rare; reduce_mask never produces such a list): the rows of a
+    // cell form a linked list.  A plain write takes the row listed last; an add sums the rows in list order.
+    if (!ADD) {
+        for (int c = ib; c >= 0; c = chain[c]) ib = max(ib, c);
+#pragma unroll
+        for (int u = 0; u < STRIP_ROWS; ++u) {
+            const bool hit = ib >= 0 && inBlock[u];
+            vec out;
+            if (hit && off[u] != BUF_OOB) out = strip_stack_load<VEC, PLANAR>(x, ib, r0 + u, s, cv, a);
+            else out = buf_load<VEC>(br, hit ? BUF_OOB : off[u]);
+            buf_store<BUF_NT>(yr, off[u], out);
+        }
+    } else {
+        int prev = -1;
+        while (ib >= 0) {
+            int cur = 0x7fffffff;
+            for (int c = ib; c >= 0; c = chain[c])
+                if (c > prev && c < cur) cur = c;
+            if (cur == 0x7fffffff) break;
+#pragma unroll
+            for (int u = 0; u < STRIP_ROWS; ++u)
+                if (inBlock[u] && off[u] != BUF_OOB) b[u] = vadd(b[u], strip_stack_load<VEC, PLANAR>(x, cur, r0 + u, s, cv, a));
+            prev = cur;
+        }
+#pragma unroll
+        for (int u = 0; u < STRIP_ROWS; ++u) buf_store<BUF_NT>(yr, off[u], b[u]);
+    }
+}
 
 struct CoverArgs {
     Geom g;
@@ -883,29 +1161,6 @@ struct CoverArgs {
 };
 
 constexpr int COVER_UNR = 4;
-
-__global__ __launch_bounds__(256) void k_cover_clear(uint32_t* __restrict__ words, int64_t n)
-{
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) words[i] = 0u;
-}
-
-// One thread per (block, block pixel): flags the pixel if it lies inside the image.  Blocks past the device-
-// resident count and rows with an image number outside [0, N) flag nothing, as they scatter nothing.
-__global__ __launch_bounds__(256) void k_cover_mark(const int16_t* __restrict__ idx, int numActive, CoverArgs a,
-                                                    uint8_t* __restrict__ flags)
-{
-    const int64_t total = (int64_t)numActive * a.RS;
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
-        const uint32_t ib = (uint32_t)(i / a.RS);
-        if (a.g.countDev && ib >= (uint32_t)*a.g.countDev) return;
-        const uint32_t p = (uint32_t)(i - (int64_t)ib * a.RS);
-        const uint32_t r = fdiv(p, a.dS), sc = p - r * (uint32_t)a.g.S;
-        const BlockOrigin o = load_origin(idx, ib, a.g);
-        const int hh = o.h0 + (int)r, ww = o.w0 + (int)sc;
-        if (o.valid && (unsigned)hh < (unsigned)a.g.H && (unsigned)ww < (unsigned)a.g.W)
-            flags[(int64_t)o.n * a.imgPixels + (int64_t)hh * a.g.W + ww] = 1;
-    }
-}
 
 // Owner map of the ordered plain scatter (SCATTER_OWNED): -1 everywhere, then the highest list position among the
 // blocks that cover each pixel.  Rows past the device-resident count and rows that name no image mark nothing.
@@ -930,23 +1185,22 @@ __global__ __launch_bounds__(256) void k_owner_mark(const int16_t* __restrict__ 
     }
 }
 
-// FLAG is the per-pixel coverage record: one byte (non-zero = covered), or the int32 owner map (>= 0 = covered).
-template <int VEC, typename FLAG>
+// Copies the pixels that no block covers (owner map entry below 0); the ordered scatter writes the others.
+template <int VEC>
 __global__ __launch_bounds__(256) void k_copy_uncovered(const float* __restrict__ src, float* __restrict__ dst,
-                                                        const FLAG* __restrict__ flags, CoverArgs a)
+                                                        const int32_t* __restrict__ owner, CoverArgs a)
 {
     typedef typename Vec<VEC>::type vec;
     const uint32_t n = blockIdx.y;
     const rsrc_t sr = make_rsrc(src + (int64_t)n * a.imgFloats, a.imgBytes);
     const rsrc_t dr = make_rsrc(dst + (int64_t)n * a.imgFloats, a.imgBytes);
-    const FLAG* __restrict__ fl = flags + (int64_t)n * a.imgPixels;
+    const int32_t* __restrict__ fl = owner + (int64_t)n * a.imgPixels;
     const uint32_t e0 = blockIdx.x * (256u * COVER_UNR) + threadIdx.x;
     bool cov[COVER_UNR];
 #pragma unroll
     for (int u = 0; u < COVER_UNR; ++u) {
         const uint32_t e = min(e0 + (uint32_t)u * 256u, a.imgV - 1u);
-        const FLAG f = fl[fdiv(e, a.dCV)];
-        cov[u] = sizeof(FLAG) == 1 ? f != 0 : (int32_t)f >= 0;
+        cov[u] = fl[fdiv(e, a.dCV)] >= 0;
     }
     uint32_t off[COVER_UNR];
 #pragma unroll
@@ -961,12 +1215,74 @@ __global__ __launch_bounds__(256) void k_copy_uncovered(const float* __restrict_
     for (int u = 0; u < COVER_UNR; ++u) buf_store<BUF_NT>(dr, off[u], v[u]);
 }
 
+// Cells that touch the image and the strip geometry; false where k_scatter_strip does not apply.
+// `planar`: the strips also stage a planar stack through LDS (strip_stage_planar); false where that does not apply.
+static bool make_strip_args(const Geom& g, int vec, bool planar, const float* x, StripArgs& a, int64_t& mapN)
+{
+    if (g.U < g.R || g.V < g.S) return false;  // overlapping blocks: a pixel may belong to several
+    a.g = g;
+    a.imgFloats = (int64_t)g.H * g.W * g.C;
+    if (a.imgFloats >= (1ll << 30)) return false;  // 32-bit byte offsets inside one image
+    if ((int64_t)g.R * g.S >= (1ll << 31)) return false;
+    auto floordiv = [](int64_t p, int64_t q) { return p >= 0 ? p / q : -((-p + q - 1) / q); };
+    int64_t bhMin = floordiv(-(int64_t)g.oh, g.U), bhMax = floordiv((int64_t)g.H - 1 - g.oh, g.U);
+    int64_t bwMin = floordiv(-(int64_t)g.ow, g.V), bwMax = floordiv((int64_t)g.W - 1 - g.ow, g.V);
+    // (cells beyond the int16 range of the list can hold no block: they stay -1 in the map)
+    if (bhMin < -(1ll << 30) || bwMin < -(1ll << 30) || bhMax > (1ll << 30) || bwMax > (1ll << 30)) return false;
+    a.bhMin = (int)bhMin; a.bwMin = (int)bwMin;
+    a.nBH = (int)(bhMax - bhMin + 1); a.nBW = (int)(bwMax - bwMin + 1);
+    mapN = (int64_t)g.N * a.nBH * a.nBW;
+    if (mapN >= (1ll << 31)) return false;
+    if ((int64_t)g.ow + (int64_t)a.bwMin * g.V < -(1ll << 31)) return false;
+    a.kPerBand = (uint32_t)((g.U + STRIP_ROWS - 1) / STRIP_ROWS);
+    a.CV = (uint32_t)(g.C / vec);
+    // NHWC stack: all channels of a pixel in one strip (both sides move whole pixels).  Planar stack: chunks of 32
+    // channels, so that a strip is wide enough in pixels to take whole cells.
+    a.CVT = planar && a.CV * (uint32_t)vec > 32u ? 32u / (uint32_t)vec : a.CV;
+    if (a.CVT > 256u) return false;
+    a.CT = a.CVT * (uint32_t)vec;
+    a.nCC = (a.CV + a.CVT - 1u) / a.CVT;
+    a.PX = 256u / a.CVT;
+    a.imgBytes = (uint32_t)(a.imgFloats * 4);
+    a.nPC = ((uint32_t)g.W + a.PX - 1u) / a.PX;
+    const int64_t tiles = (int64_t)g.N * a.nBH * a.kPerBand * a.nPC * a.nCC;
+    if (tiles >= (1ll << 31)) return false;
+    a.tiles = (uint32_t)tiles;
+    a.swzMask = 0;
+    a.S4 = 1;
+    a.cellsPerStrip = 1;
+    if (planar) {
+        // strips that line up with the cells, planar rows that are whole 16-byte vectors (see strip_stage_planar)
+        if (g.S % 4 != 0 || g.V % 4 != 0 || (uint32_t)g.V > a.PX || a.PX % (uint32_t)g.V != 0) return false;
+        if (g.ow + a.bwMin * g.V != 0 || (reinterpret_cast<uintptr_t>(x) & 15) != 0) return false;
+        a.S4 = (uint32_t)g.S / 4u;
+        a.cellsPerStrip = a.PX / (uint32_t)g.V;
+        if (a.CT % 4u == 0) {
+            const uint32_t c4 = a.CT / 4u, low = c4 & (~c4 + 1u);  // largest power of two that divides CT/4
+            a.swzMask = (low > 8u ? 8u : low) - 1u;
+        }
+    }
+    a.dCVT = make_fastdiv(a.CVT);
+    a.dCC = make_fastdiv(a.nCC);
+    a.dV = make_fastdiv((uint32_t)g.V);
+    a.dK = make_fastdiv(a.kPerBand);
+    a.dPC = make_fastdiv(a.nPC);
+    a.dBH = make_fastdiv((uint32_t)a.nBH);
+    a.dS4 = make_fastdiv(a.S4);
+    a.dCT = make_fastdiv(a.CT);
+    return true;
+}
+
+// Scratch of the one-pass copying scatter: the cell map, the duplicate flag, one chain entry per list row.
 size_t scatter_cover_workspace_bytes(const Geom& g, int numActive)
 {
     if (numActive <= 0) return 0;
-    if ((int64_t)g.H * g.W * g.C >= (1ll << 30)) return 0;  // 32-bit byte offsets inside one image
-    if ((int64_t)g.R * g.S >= (1ll << 31)) return 0;
-    return (((size_t)g.N * g.H * g.W + 3) & ~(size_t)3) + 16;
+    StripArgs a;
+    int64_t mapN = 0;
+    // (with the widest channel vectors C allows; a call whose pointers force narrower ones checks again)
+    if (make_strip_args(g, g.C % 4 == 0 ? 4 : (g.C % 2 == 0 ? 2 : 1), false, nullptr, a, mapN))
+        return (size_t)mapN * 4 + 16 + (size_t)numActive * 4 + 16;
+    return 0;
 }
 
 static void make_cover_args(const Geom& g, int vec, CoverArgs& c)
@@ -1083,49 +1399,83 @@ hipError_t launch_scatter_owned(const float* x, float* y, const int16_t* idx, in
     return scatter_from(x, y, y, idx, numActive, g, transpose, SCATTER_ASSIGN, stream, owner);
 }
 
+template <int VEC>
+static void launch_strip(const float* x, const float* ybase, float* y, bool planar, int op, const int32_t* map,
+                         const int32_t* chain, const int32_t* dup, const StripArgs& a, hipStream_t stream)
+{
+    const dim3 grid(a.tiles);
+    const size_t lds = planar ? (size_t)STRIP_ROWS * a.PX * a.CT * sizeof(float) : 0;  // 16 KB with 16-byte vectors
+#define SBNET_STRIP(OP, PL) \
+    hipLaunchKernelGGL((k_scatter_strip<VEC, OP, PL>), grid, dim3(256), lds, stream, x, ybase, y, map, chain, dup, a)
+    if (op == STRIP_COPY) SBNET_STRIP(STRIP_COPY, false);
+    else if (op == STRIP_ADD && planar) SBNET_STRIP(STRIP_ADD, true);
+    else if (op == STRIP_ADD) SBNET_STRIP(STRIP_ADD, false);
+    else if (planar) SBNET_STRIP(STRIP_ASSIGN, true);
+    else SBNET_STRIP(STRIP_ASSIGN, false);
+#undef SBNET_STRIP
+}
+
 hipError_t launch_scatter_over_base(const float* x, const float* ybase, float* y, const int16_t* idx, int numActive,
                                     const Geom& g, bool transpose, ScatterMode mode, void* workspace,
                                     size_t workspaceBytes, hipStream_t stream, bool& done)
 {
     done = false;
     if (mode == SCATTER_ATOMIC || numActive <= 0) return hipSuccess;
-    const size_t need = scatter_cover_workspace_bytes(g, numActive);
-    if (!workspace || need == 0 || workspaceBytes < need || (reinterpret_cast<uintptr_t>(workspace) & 3))
-        return hipSuccess;
-    // Two small launches prepare the flags: worth it once the blocks cover enough of the tensor to pay for them
-    // (each covered byte saves one read and one write of the copy).
-    if ((int64_t)numActive * g.R * g.S * g.C * 4 < (16ll << 20)) return hipSuccess;
+    if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 3)) return hipSuccess;
 
+    // Blocks that do not overlap: one streaming pass over the output (k_scatter_strip).  A planar stack whose
+    // geometry the strips do not stage is scattered by the tile kernel after a pass that copies the rest.
+    {
+        StripArgs a;
+        int64_t mapN = 0;
+        const int vb = pick_vec(g, ybase, y), vx = pick_vec(g, transpose ? nullptr : x, nullptr);
+        const int vec = vb < vx ? vb : vx;
+        const size_t need = scatter_cover_workspace_bytes(g, numActive);
+        bool planar = transpose;
+        bool ok = need != 0 && workspaceBytes >= need;
+        if (ok && !make_strip_args(g, vec, planar, x, a, mapN)) {
+            planar = false;
+            // (two passes and four launches: worth it once the blocks cover enough of the tensor)
+            ok = transpose && (int64_t)numActive * g.R * g.S * g.C * 4 >= (16ll << 20) &&
+                 make_strip_args(g, vec, false, x, a, mapN);
+        }
+        if (ok) {
+            a.g = g;
+            int32_t* map = static_cast<int32_t*>(workspace);
+            int32_t* dup = map + mapN;
+            int32_t* chain = dup + 4;
+            int64_t fillWgs = (mapN + 255) / 256;
+            if (fillWgs > 4096) fillWgs = 4096;
+            hipLaunchKernelGGL(k_pull_fill, dim3((unsigned)fillWgs), dim3(256), 0, stream, map, mapN, dup);
+            hipLaunchKernelGGL(k_cell_map, dim3((unsigned)((numActive + 255) / 256)), dim3(256), 0, stream, idx, numActive,
+                               a, map, chain, dup);
+            const int op = transpose && !planar ? STRIP_COPY : (mode == SCATTER_ADD ? STRIP_ADD : STRIP_ASSIGN);
+            if (vec == 4) launch_strip<4>(x, ybase, y, planar, op, map, chain, dup, a, stream);
+            else if (vec == 2) launch_strip<2>(x, ybase, y, planar, op, map, chain, dup, a, stream);
+            else launch_strip<1>(x, ybase, y, planar, op, map, chain, dup, a, stream);
+            done = true;
+            if (op == STRIP_COPY) return scatter_from(x, y, ybase, idx, numActive, g, transpose, mode, stream);
+            return hipGetLastError();
+        }
+    }
+
+    // Plain writes of overlapping blocks: the owner map of the ordered scatter also tells which pixels are covered.
+    // Two small launches prepare it: worth it once the blocks cover enough of the tensor to pay for them (each
+    // covered byte saves one read and one write of the copy).
+    if (mode != SCATTER_ASSIGN || scatter_owner_workspace_bytes(g, numActive) == 0) return hipSuccess;
+    if ((int64_t)numActive * g.R * g.S * g.C * 4 < (16ll << 20)) return hipSuccess;
+    if ((int64_t)g.H * g.W * g.C >= (1ll << 30)) return hipSuccess;  // 32-bit byte offsets inside one image
     CoverArgs c;
     const int vec = pick_vec(g, ybase, y);
     make_cover_args(g, vec, c);
     const dim3 grid((c.imgV + 256u * COVER_UNR - 1) / (256u * COVER_UNR), (unsigned)g.N);
-
-    // Plain writes of overlapping blocks: the owner map of the ordered scatter also tells which pixels are covered.
-    if (mode == SCATTER_ASSIGN && scatter_owner_workspace_bytes(g, numActive) != 0) {
-        int32_t* owner = nullptr;
-        if (!build_owner_map(idx, numActive, g, workspace, workspaceBytes, stream, owner)) return hipSuccess;
-        if (vec == 4) hipLaunchKernelGGL((k_copy_uncovered<4, int32_t>), grid, dim3(256), 0, stream, ybase, y, owner, c);
-        else if (vec == 2) hipLaunchKernelGGL((k_copy_uncovered<2, int32_t>), grid, dim3(256), 0, stream, ybase, y, owner, c);
-        else hipLaunchKernelGGL((k_copy_uncovered<1, int32_t>), grid, dim3(256), 0, stream, ybase, y, owner, c);
-        done = true;
-        return scatter_from(x, y, ybase, idx, numActive, g, transpose, mode, stream, owner);
-    }
-    uint8_t* flags = static_cast<uint8_t*>(workspace);
-
-    const int64_t words = (int64_t)((need - 16) / 4);
-    int64_t wgs = (words + 255) / 256;
-    if (wgs > 8192) wgs = 8192;
-    hipLaunchKernelGGL(k_cover_clear, dim3((unsigned)wgs), dim3(256), 0, stream, reinterpret_cast<uint32_t*>(flags), words);
-    int64_t markWgs = ((int64_t)numActive * c.RS + 255) / 256;
-    if (markWgs > 65536) markWgs = 65536;
-    hipLaunchKernelGGL(k_cover_mark, dim3((unsigned)markWgs), dim3(256), 0, stream, idx, numActive, c, flags);
-    const uint8_t* cflags = flags;
-    if (vec == 4) hipLaunchKernelGGL((k_copy_uncovered<4, uint8_t>), grid, dim3(256), 0, stream, ybase, y, cflags, c);
-    else if (vec == 2) hipLaunchKernelGGL((k_copy_uncovered<2, uint8_t>), grid, dim3(256), 0, stream, ybase, y, cflags, c);
-    else hipLaunchKernelGGL((k_copy_uncovered<1, uint8_t>), grid, dim3(256), 0, stream, ybase, y, cflags, c);
+    int32_t* owner = nullptr;
+    if (!build_owner_map(idx, numActive, g, workspace, workspaceBytes, stream, owner)) return hipSuccess;
+    if (vec == 4) hipLaunchKernelGGL((k_copy_uncovered<4>), grid, dim3(256), 0, stream, ybase, y, owner, c);
+    else if (vec == 2) hipLaunchKernelGGL((k_copy_uncovered<2>), grid, dim3(256), 0, stream, ybase, y, owner, c);
+    else hipLaunchKernelGGL((k_copy_uncovered<1>), grid, dim3(256), 0, stream, ybase, y, owner, c);
     done = true;
-    return scatter_from(x, y, ybase, idx, numActive, g, transpose, mode, stream);
+    return scatter_from(x, y, ybase, idx, numActive, g, transpose, mode, stream, owner);
 }
 
 hipError_t launch_copy(float* dst, const float* src, size_t count, hipStream_t stream)

@@ -547,6 +547,40 @@ def test_copying_scatter_moves_every_byte_once(geom):
     np.testing.assert_array_equal(host(y3), y_o)
 
 
+@pytest.mark.parametrize("geom", [
+    # (N, H, W, C), bsize, bstride, boffset
+    ((2, 40, 56, 32), (4, 4), (4, 4), (0, 0)),      # whole 4x4 planes: the planar stack is staged through LDS
+    ((1, 64, 64, 64), (8, 8), (8, 8), (-3, 0)),     # two channel chunks, rows offset
+    ((2, 30, 44, 16), (3, 4), (5, 8), (1, 0)),      # gaps between the blocks
+    ((1, 33, 47, 5), (5, 7), (6, 7), (-2, -3)),     # scalar channel vectors, nothing aligned
+])
+def test_copying_scatter_of_a_list_with_repeated_rows(geom):
+    """Non-overlapping blocks, a list that names some blocks twice or three times with different stack rows: the
+    sequential CPU functor lets the last row win a plain write and adds every row, in list order, for add=True
+    (sparse_gather.cc:105-129).  The copying op (built in one pass over the output) does the same, bit for bit."""
+    (N, H, W, C), bs, bst, bo = geom
+    rng = np.random.default_rng(H + W + C)
+    bc = bcount_covering(H, W, bst, bo)
+    cells = [(n, i, j) for n in range(N) for i in range(bc[0]) for j in range(bc[1]) if rng.random() < 0.6]
+    idx = np.array(cells + cells[:5] + cells[2:4], np.int16)
+    rng.shuffle(idx, axis=0)
+    M = len(idx)
+    cnt = np.array([M], np.int32)
+    base = rng.standard_normal((N, H, W, C)).astype(np.float32)
+    aligned = bs[1] % 4 == 0 and bst[1] % 4 == 0 and bo[1] % bst[1] == 0
+    for transpose in ((False, True) if aligned else (False,)):
+        shape = (M, C, bs[0], bs[1]) if transpose else (M, bs[0], bs[1], C)
+        stack = (rng.standard_normal(shape) * rng.choice([1e-3, 1.0, 1e4], size=(M, 1, 1, 1))).astype(np.float32)
+        for add in (False, True):
+            y_o = orc.sparse_scatter(stack, cnt, idx, base, bs, bst, bo, add=add, transpose=transpose)
+            y = sbnet_amd.sparse_scatter(dev(stack), cnt, dev(idx), dev(base), bs, bst, bo, add=add, transpose=transpose)
+            np.testing.assert_array_equal(host(y), y_o, err_msg="transpose %s add %s" % (transpose, add))
+            dcount = torch.tensor([M - 3], dtype=torch.int32, device=DEV)
+            y_o2 = orc.sparse_scatter(stack, [M - 3], idx, base, bs, bst, bo, add=add, transpose=transpose)
+            y = sbnet_amd.sparse_scatter(dev(stack), dcount, dev(idx), dev(base), bs, bst, bo, add=add, transpose=transpose)
+            np.testing.assert_array_equal(host(y), y_o2, err_msg="device count, transpose %s add %s" % (transpose, add))
+
+
 @pytest.mark.parametrize("case", [
     # (H, W, C), bsize, bstride, boffset, block list (n, bh, bw)
     ((20, 30, 8), (6, 7), (6, 7), (0, 0), []),                                   # empty list
