@@ -102,7 +102,9 @@ size_t sbnet_reduce_mask_workspace_bytes(int N, const int32_t* bcount, int bcoun
  *   (reduce_mask.cc:206-218); the fix-up happens on the device, without a host round trip.
  *   workspace             device scratch of sbnet_reduce_mask_workspace_bytes() bytes, 16-byte
  *                         aligned, or NULL to let the call allocate and free its own
- *                         (slower, and it synchronises the stream).
+ *                         (slower, and it synchronises the stream; refused with SBNET_EHIP /
+ *                         hipErrorStreamCaptureUnsupported, before anything is allocated or enqueued,
+ *                         while `stream` is being captured).
  */
 int sbnet_reduce_mask(const float* mask, int N, int H, int W,
                       const int32_t* bcount, int bcount_len,
@@ -128,6 +130,9 @@ int sbnet_reduce_mask(const float* mask, int N, int H, int W,
  *   streams, different threads) race on it and must be serialised by the caller; calls on one stream are.
  *   Nothing in the array has to be cleared between calls (every byte of it that a call reads has been
  *   written by that call), so a smaller problem may follow a larger one.
+ *   The first call on a device looks the array's device address up (hipGetSymbolAddress, once per device, under
+ *   a mutex): make that call outside stream capture; every later call does no HIP call but its kernel launches
+ *   and may be captured.
  */
 int sbnet_reduce_mask_static(const float* mask, int N, int H, int W,
                              const int32_t* bcount, int bcount_len,
@@ -282,11 +287,15 @@ int sbnet_sparse_scatter_functor_ws(const float* x, int N, int H, int W, int C, 
                                     void* workspace, size_t workspace_bytes, void* stream);
 
 /* Library-managed device scratch for callers that have no allocator at hand (the functor level of the reference
-   passes none down, sparse_gather.h:45-66): returns a buffer of at least `bytes` bytes on the current device that
-   stays valid until the next sbnet_scratch_acquire on the same stream or sbnet_shutdown.  One grow-only buffer is
-   kept per (device, stream); calls on one stream run in order, so they may share it.  Growing allocates (and
-   waits for the stream); a request that would have to grow while `stream` is being captured returns NULL, as does
-   a failed allocation.  Thread-safe. */
+   passes none down, sparse_gather.h:45-66): returns a buffer of at least `bytes` bytes on the current device.  One
+   grow-only buffer is kept per (device, stream); calls on one stream run in order, so consecutive calls of ONE
+   host thread on that stream may share it: the pointer is good for the library calls that thread makes next on
+   that stream, until its next sbnet_scratch_acquire there.  The bookkeeping is thread-safe and no buffer is
+   freed before sbnet_shutdown (a buffer that has been outgrown is kept until then, so a pointer handed out
+   earlier never dangles), but two host threads that enqueue on the same stream would interleave their launches
+   over the one buffer and corrupt each other's scratch: one enqueuing thread per stream, or scratch of the
+   caller's own per call (a TensorFlow binding: allocate_temp).  Growing allocates; a request that would have
+   to grow while `stream` is being captured returns NULL, as does a failed allocation. */
 void* sbnet_scratch_acquire(size_t bytes, void* stream);
 
 /* Frees what the library keeps between calls: the buffers of sbnet_scratch_acquire and the pinned count words of

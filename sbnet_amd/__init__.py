@@ -8,12 +8,12 @@ and raises if it has not been built.
 """
 from .block_params import (BlockParams, calc_block_params, calc_block_params_res_block,  # noqa: F401
                            calc_block_count_covering)
-from .ops import (HipError, InvalidArgument, ReduceMaskResult, reduce_mask, sparse_gather,  # noqa: F401
-                  sparse_scatter, sparse_scatter_var)
+from .ops import (HipError, InvalidArgument, ReduceMaskResult, reduce_mask, release_workspaces,  # noqa: F401
+                  sparse_gather, sparse_scatter, sparse_scatter_var)
 from .autograd import SparseGatherFunction, SparseScatterFunction  # noqa: F401
 
 __all__ = [
     "reduce_mask", "sparse_gather", "sparse_scatter", "sparse_scatter_var", "ReduceMaskResult",
-    "InvalidArgument", "HipError", "SparseGatherFunction", "SparseScatterFunction", "BlockParams", "calc_block_params", "calc_block_params_res_block",
+    "InvalidArgument", "HipError", "release_workspaces", "SparseGatherFunction", "SparseScatterFunction", "BlockParams", "calc_block_params", "calc_block_params_res_block",
     "calc_block_count_covering",
 ]

@@ -183,27 +183,26 @@ int reduce_mask_impl(const float* mask, int N, int H, int W, const int32_t* bcou
     const size_t need = sbnet::reduce_mask_workspace_bytes(T);
     void* ws = workspace;
     bool ownWs = false;
-    if (ws) {
-        if (workspaceBytes < need || (reinterpret_cast<uintptr_t>(ws) & 15)) return SBNET_EINVAL_ARG;
-    } else {
+    if (ws && (workspaceBytes < need || (reinterpret_cast<uintptr_t>(ws) & 15))) return SBNET_EINVAL_ARG;
+    // Neither a host-visible count (nothing runs during capture) nor a scratch buffer of the library's own
+    // (allocating and freeing it synchronises) can be had while the stream is being captured: refuse before
+    // anything is allocated or enqueued, so the capture stays valid.
+    bool capturing = false;
+    if (countHost || !ws) {
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &cap) != hipSuccess) (void)hipGetLastError();  // (cannot be asked: not capturing)
+        else capturing = cap != hipStreamCaptureStatusNone;
+        if (capturing) return hip_fail(hipErrorStreamCaptureUnsupported);
+    }
+    if (!ws) {
         SBNET_HIP(hipMalloc(&ws, need));
         ownWs = true;
     }
     const sbnet::Geom g = make_geom(N, H, W, 1, bsize, bstride, boffset);
-    // a host-visible count cannot be produced while the stream is being captured (nothing runs): refuse before
-    // anything is enqueued, so the capture stays valid
     HostSignal* sig = nullptr;
     uint32_t seq = 0;
     if (countHost) {
-        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-        if (hipStreamIsCapturing(stream, &cap) != hipSuccess) {
-            (void)hipGetLastError();
-        } else if (cap != hipStreamCaptureStatusNone) {
-            if (ownWs) (void)hipFree(ws);
-            return hip_fail(hipErrorStreamCaptureUnsupported);
-        } else {
-            sig = host_signal();
-        }
+        sig = host_signal();
         if (sig) {
             seq = ++sig->seq;
             if (seq == 0) seq = ++sig->seq;  // 0 is the word's initial tag
@@ -289,6 +288,10 @@ struct ScratchSlot {
 };
 std::mutex g_scratchMutex;
 std::vector<ScratchSlot> g_scratch;
+// Buffers that a slot has outgrown.  A caller may still hold such a pointer (it asked before another thread's
+// larger request on the same stream) and work that uses it may still be queued, so nothing is freed before
+// sbnet_shutdown.
+std::vector<ScratchSlot> g_scratchRetired;
 
 }  // namespace
 
@@ -352,9 +355,12 @@ int sbnet_reduce_mask_static(const float* mask, int N, int H, int W, const int32
         !pair_ok(boffset, boffset_len))
         return SBNET_EINVAL_PARAM_SHAPE;
     if (!bin_counts_device) return SBNET_EINVAL_ARG;
-    const int64_t T = sbnet_reduce_mask_max_indices(N, bcount, bcount_len);
-    if (T < 0 || T >= (1ll << 31) || sbnet::reduce_mask_workspace_bytes(T) > sbnet::STATIC_SCRATCH_BYTES)
-        return SBNET_ETOOBIG;
+    // what sbnet_reduce_mask rejects as an argument error is one here too; SBNET_ETOOBIG is for valid sizes only
+    if (N <= 0 || bcount[0] <= 0 || bcount[1] <= 0 || N > 32768 || bcount[0] > 32768 || bcount[1] > 32768)
+        return SBNET_EINVAL_ARG;
+    const int64_t T = (int64_t)N * bcount[0] * bcount[1];
+    if (T >= (1ll << 31)) return SBNET_EINVAL_ARG;
+    if (sbnet::reduce_mask_workspace_bytes(T) > sbnet::STATIC_SCRATCH_BYTES) return SBNET_ETOOBIG;
     void* ws = nullptr;
     SBNET_HIP(sbnet::static_scratch(&ws));
     return reduce_mask_impl(mask, N, H, W, bcount, bsize, bstride, boffset, tol, avgpool, true, active_block_indices,
@@ -597,9 +603,7 @@ void* sbnet_scratch_acquire(size_t bytes, void* stream)
         return nullptr;
     }
     if (slot) {
-        // the old buffer may still be in use by work queued on the stream
-        (void)hipStreamSynchronize(s);
-        (void)hipFree(slot->ptr);
+        g_scratchRetired.push_back(*slot);  // may still be handed out or in use by queued work: kept until shutdown
         slot->ptr = p;
         slot->bytes = want;
     } else {
@@ -613,15 +617,17 @@ int sbnet_shutdown(void)
     hipError_t first = hipSuccess;
     {
         std::lock_guard<std::mutex> lock(g_scratchMutex);
-        for (ScratchSlot& c : g_scratch) {
-            int cur = 0;
-            (void)hipGetDevice(&cur);
-            (void)hipSetDevice(c.dev);
-            hipError_t e = hipFree(c.ptr);  // waits for the device
-            (void)hipSetDevice(cur);
-            if (e != hipSuccess && first == hipSuccess) first = e;
+        for (std::vector<ScratchSlot>* list : {&g_scratch, &g_scratchRetired}) {
+            for (ScratchSlot& c : *list) {
+                int cur = 0;
+                (void)hipGetDevice(&cur);
+                (void)hipSetDevice(c.dev);
+                hipError_t e = hipFree(c.ptr);  // waits for the device
+                (void)hipSetDevice(cur);
+                if (e != hipSuccess && first == hipSuccess) first = e;
+            }
+            list->clear();
         }
-        g_scratch.clear();
     }
     {
         // only the words no thread holds; a live thread keeps its own until it ends

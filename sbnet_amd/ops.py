@@ -112,6 +112,15 @@ def _workspace(device, nbytes):
     return ws
 
 
+def release_workspaces():
+    """Drops the scratch buffers the op wrappers keep per (device, stream) between calls (they only ever grow) and
+    the library's own (sbnet_shutdown).  Waits for the device; the ops can be used again afterwards."""
+    if _workspaces:
+        torch.cuda.synchronize()
+    _workspaces.clear()
+    _check(_lib.load().sbnet_shutdown())
+
+
 def _param(dynamic, attr, name):
     """The ops take their block parameters as `dynamic_b*` inputs (reduce_mask.cc:100-110, sparse_gather.cc:48-57);
     the reference's README.md:53-107 and sample.py:42-43 spell the same int pairs `bsize=`, `bstride=`, `boffset=`

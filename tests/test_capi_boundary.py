@@ -105,13 +105,18 @@ def test_size_queries():
 def test_scatter_workspace_query():
     lib = _lib.load()
     dims = I64x4(2, 512, 512, 256)
-    flags = 2 * 512 * 512 + 16   # one flag byte per pixel: the copying scatter built in one pass
+    # the copying scatter built in one pass: one int32 per cell of the block grid, a flag, one int32 per list row
+    cells = 2 * 32 * 32 * 4 + 16 + 2000 * 4 + 16
     owner = 2 * 512 * 512 * 4 + 16  # one int32 per pixel: overlapping plain writes in the CPU functor's order
-    # blocks that tile (stride == size): no order is needed; the flag bytes, or the block tables of the atomic-free add
+    # blocks that tile (stride == size): no order is needed; the cell map, or the block tables of the atomic-free add
     # (which also serves atomic=1 on tiling blocks) if those are larger
     tables = 2 * 32 * 32 * 4 + 32 + 2000 * 72 * 4
     assert lib.sbnet_sparse_scatter_workspace_bytes(2000, dims, 4, I32x2(16, 16), 2, I32x2(16, 16), 2, I32x2(0, 0),
-                                                    2) == max(flags, tables)
+                                                    2) == max(cells, tables)
+    # gaps between the blocks, few of them: the same two candidates
+    assert lib.sbnet_sparse_scatter_workspace_bytes(10, dims, 4, I32x2(5, 7), 2, I32x2(16, 16), 2, I32x2(0, 0),
+                                                    2) == max(2 * 32 * 32 * 4 + 16 + 10 * 4 + 16,
+                                                              2 * 32 * 32 * 4 + 32 + 10 * 72 * 4)
     # 16x16 blocks at stride 8: 2x2 blocks cover a pixel, the atomic-free add applies
     n = lib.sbnet_sparse_scatter_workspace_bytes(2000, dims, 4, I32x2(16, 16), 2, I32x2(8, 8), 2, I32x2(0, 0), 2)
     assert n >= max(2 * 64 * 64 * 4 + 2000 * 4, owner)
@@ -238,6 +243,39 @@ def test_python_mirror_checks_sizes_before_any_launch():
                              ((5, 3, 4), False)):        # not rank 4
         with pytest.raises(ops.InvalidArgument, match="block stack of shape"):
             ops._check_stack(torch.zeros(shape), 5, 8, 3, 4, transpose, "x")
+
+
+@pytest.mark.gpu
+def test_scratch_provider_keeps_outgrown_buffers_until_shutdown():
+    """sbnet_scratch_acquire hands one grow-only buffer per stream to callers without an allocator.  A pointer it
+    has handed out stays valid when a later, larger request on the same stream replaces the buffer (another thread
+    may have asked in between): the outgrown buffer is kept until sbnet_shutdown.  release_workspaces() drops the
+    Python mirror's buffers as well, and the ops work again afterwards."""
+    import numpy as np
+    import torch
+    import sbnet_amd
+    lib = _lib.load()
+    assert lib.sbnet_shutdown() == 0
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    small = lib.sbnet_scratch_acquire(1 << 20, stream)
+    assert small and lib.sbnet_scratch_acquire(4096, stream) == small     # fits: the same buffer
+    src = torch.arange(1 << 18, dtype=torch.float32, device="cuda:0")
+    large = lib.sbnet_scratch_acquire(8 << 20, stream)                    # grows: a new buffer
+    assert large and large != small
+    # the first pointer is still device memory the caller may use (work queued on it may not have run yet)
+    assert lib.sbnet_copy_tensor(small, src.data_ptr(), 1 << 18, stream) == 0
+    back = torch.empty_like(src)
+    assert lib.sbnet_copy_tensor(back.data_ptr(), small, 1 << 18, stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(back, src)
+    assert lib.sbnet_scratch_acquire(2 << 20, stream) == large
+    free_before = torch.cuda.mem_get_info()[0]
+    sbnet_amd.release_workspaces()                                         # sbnet_shutdown inside
+    assert torch.cuda.mem_get_info()[0] >= free_before + (8 << 20)
+    mask = torch.ones((1, 8, 8, 1), device="cuda:0")
+    r = sbnet_amd.reduce_mask(mask, [2, 2], [4, 4], [4, 4], [0, 0], tol=0.5)
+    assert int(r.bin_counts[0]) == 4
+    assert np.array_equal(r.active_block_indices.cpu().numpy()[:4], [[0, 0, 0], [0, 0, 1], [0, 1, 0], [0, 1, 1]])
 
 
 def test_python_mirror_fails_loudly_without_library(monkeypatch):
