@@ -365,6 +365,7 @@ struct TileFixed {
     static constexpr uint32_t kPp = (P_ + 31) / 32 * 32;
     static constexpr uint32_t kVpr = (P_ + 3) / 4;
     static constexpr uint32_t kCchunks = (C_ + 4 * kLpp - 1) / (4 * kLpp);
+    static constexpr uint32_t kNthr = NTHR_, kCt = 4 * kLpp;
     __host__ __device__ static constexpr uint32_t nthr(const TileArgs&) { return NTHR_; }
     __host__ __device__ static constexpr uint32_t S(const TileArgs&) { return S_; }
     __host__ __device__ static constexpr uint32_t C(const TileArgs&) { return C_; }

@@ -294,6 +294,135 @@ __device__ __forceinline__ void scatter_planar_tile(const float* __restrict__ x,
     }
 }
 
+// The same tile moved in two halves, for launches of so few workgroups that all of them are resident at once: such
+// a launch runs in lockstep (every workgroup loads, then every workgroup stores), so its reads and its writes do
+// not overlap and it takes the sum of both.  Here a workgroup issues the loads of both halves of its pixels up
+// front, and stores the first half (the first 2 of a thread's 4 NHWC pixels: 2 * nthr / 8 tile pixels) while the
+// second half's loads are still arriving.  Fixed-shape instances of plain and ordered writes only (4-float channel
+// vectors, full channel chunks, every split at least as long as the first half).
+template <int MODE, typename G>
+__device__ __forceinline__ void scatter_planar_tile_halves(const float* __restrict__ x, float* y,
+                                                           const int16_t* __restrict__ idx, const TileArgs& a,
+                                                           float* lds, uint32_t* waveBits, uint32_t ib, uint32_t rem)
+{
+    constexpr uint32_t nthr = G::kNthr, RS = G::kRS, Pp = G::kPp, vpr = G::kVpr;
+    constexpr uint32_t PA = 2u * (nthr >> G::kLppLog);  // pixels of the first half
+    constexpr uint32_t vprA = PA / 4u, vprB = vpr - vprA;
+    constexpr uint32_t CT = G::kCt;
+    static_assert(CT * vprA == 2u * nthr, "two loads per thread cover the first half");
+    static_assert(CT * vprB <= nthr && vprB > 0, "one load per thread covers the second half");
+    const uint32_t tid = threadIdx.x;
+    TileId t;
+    decode_tile<G>(a, t, ib, rem);
+    const RawTriple raw = load_triple(idx, t.ib);
+    if (beyond_count(a.g, t.ib)) return;
+    const rsrc_t xr = make_rsrc(x + ((int64_t)t.ib * G::C(a) + t.c0) * RS + t.p0,
+                                ((uint32_t)(t.ctEff - 1) * RS + (uint32_t)t.Pn) * 4u);
+    f4 valA[2], valB;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+        const uint32_t i = (uint32_t)u * nthr + tid;
+        valA[u] = buf_load<4>(xr, ((i / vprA) * RS + 4u * (i % vprA)) * 4u);
+    }
+    const uint32_t cB = tid / vprB, eB = vprA + tid % vprB;
+    const int e0B = min(4 * (int)eB, t.Pn - 4);  // a partial last slot is read as the run's last 4 floats
+    valB = buf_load<4>(xr, cB < CT ? (cB * RS + (uint32_t)e0B) * 4u : BUF_OOB);
+    ListRow rows[RANK_ROWS_PER_THREAD];
+    uint32_t listCount = 0;
+    ListRows lr;
+    if (MODE == SCATTER_RANKED_INLINE) {
+        listCount = list_count(a.g, a.blocks);
+        lr = list_rows(idx, listCount);
+#pragma unroll
+        for (int u = 0; u < RANK_ROWS_PER_THREAD; ++u) {
+            const uint32_t j = t.ib + 1u + (uint32_t)u * nthr + tid;
+            rows[u] = list_row_load(lr, j, j < listCount);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+        const uint32_t i = (uint32_t)u * nthr + tid;
+        const uint32_t c = i / vprA;
+        *reinterpret_cast<f4*>(lds + c * Pp + ((4u * (i % vprA)) ^ lds_swz(c))) = valA[u];
+    }
+    const BlockOrigin o = origin_of(raw, a.g);
+    if (MODE == SCATTER_RANKED_INLINE) {
+        uint32_t bits = 0u;
+#pragma unroll
+        for (int u = 0; u < RANK_ROWS_PER_THREAD; ++u) {
+            int n2, bh2, bw2;
+            list_row_unpack(rows[u], n2, bh2, bw2);
+            if (t.ib + 1u + (uint32_t)u * nthr + tid < listCount) bits |= rank_pair_bits(o.n, o.bh, o.bw, n2, bh2, bw2);
+        }
+        for (uint32_t j = t.ib + 1u + (uint32_t)RANK_ROWS_PER_THREAD * nthr + tid; j < listCount; j += nthr) {
+            int n2, bh2, bw2;
+            list_row_unpack(list_row_load(lr, j, true), n2, bh2, bw2);
+            bits |= rank_pair_bits(o.n, o.bh, o.bw, n2, bh2, bw2);
+        }
+        if (__ballot(bits != 0u) != 0ull)
+            for (int off = 32; off > 0; off >>= 1) bits |= (uint32_t)__shfl_xor((int)bits, off);
+        if ((tid & 63u) == 0u) waveBits[tid >> 6] = bits;
+    }
+    lds_barrier();
+    if (!o.valid) return;   // (the whole workgroup)
+    const rsrc_t yr = make_rsrc(y + (int64_t)o.n * a.imgFloats, a.imgBytes);
+    const uint32_t c0l = (tid & ((1u << G::kLppLog) - 1u)) * 4u;
+    uint32_t rbits = 0u;
+    if (MODE == SCATTER_RANKED_INLINE) {
+        for (uint32_t w = 0; w < (nthr >> 6); ++w) rbits |= waveBits[w];
+    }
+    uint32_t offs[TILE_LD], pls[TILE_LD];
+    nhwc_walk<4, G>(a, t, o, tid, nthr, [&](int u, uint32_t pl, uint32_t off, uint32_t, uint32_t r, uint32_t sc) {
+        if (MODE == SCATTER_RANKED_INLINE && ranked_out(rbits, r, sc, a.g)) off = BUF_OOB;
+        offs[u] = off;
+        pls[u] = pl;
+    });
+    auto store_items = [&](int u0) {
+        f4 w[2];
+#pragma unroll
+        for (int v = 0; v < 2; ++v) {
+            const int u = u0 + v;
+            w[v] = (f4)(0.f);
+            if (offs[u] != BUF_OOB) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t c = c0l + (uint32_t)k;
+                    vset(w[v], k, lds[c * Pp + (pls[u] ^ lds_swz(c))]);
+                }
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < 2; ++v) buf_store<BUF_NT>(yr, offs[u0 + v], w[v]);
+    };
+    store_items(0);
+    // second half: its loads were issued before the first half's stores and complete before them
+    if (cB < CT) {
+        float* __restrict__ row = lds + cB * Pp;
+        if (4 * (int)eB + 4 <= t.Pn) {
+            *reinterpret_cast<f4*>(row + ((4u * eB) ^ lds_swz(cB))) = valB;
+        } else if (4 * (int)eB < t.Pn) {
+            const uint32_t t0 = (uint32_t)(t.Pn - 4);
+            row[(t0 + 0) ^ lds_swz(cB)] = valB.x;
+            row[(t0 + 1) ^ lds_swz(cB)] = valB.y;
+            row[(t0 + 2) ^ lds_swz(cB)] = valB.z;
+            row[(t0 + 3) ^ lds_swz(cB)] = valB.w;
+        }
+    }
+    lds_barrier();
+    store_items(2);
+}
+
+// Geometry policy of the tile moved in two halves (same tile as TileFixed).
+template <int R_, int S_, int C_, int P_, int NTHR_>
+struct TileFixedHalves : TileFixed<R_, S_, C_, P_, NTHR_> {
+    static constexpr bool HALVES = true;
+};
+
+template <typename G, typename = void>
+struct tile_in_halves { static constexpr bool value = false; };
+template <typename G>
+struct tile_in_halves<G, decltype((void)G::HALVES)> { static constexpr bool value = G::HALVES; };
+
 template <int VEC, int MODE, typename G>
 __global__ __launch_bounds__(512) void k_scatter_planar(const float* __restrict__ x, float* y, const float* ysrc,
                                                         const int16_t* __restrict__ idx, TileArgs a, ColorArgs col)
@@ -301,7 +430,10 @@ __global__ __launch_bounds__(512) void k_scatter_planar(const float* __restrict_
     extern __shared__ __attribute__((aligned(16))) float lds[];
     __shared__ uint32_t waveBits[8];  // SCATTER_RANKED_INLINE: one word per wave
     for_each_block_of_workgroup(a, G::tpb(a), [&](uint32_t ib, uint32_t rem) {
-        scatter_planar_tile<VEC, MODE, G>(x, y, ysrc, idx, a, col, lds, waveBits, ib, rem);
+        if constexpr (tile_in_halves<G>::value)
+            scatter_planar_tile_halves<MODE, G>(x, y, idx, a, lds, waveBits, ib, rem);
+        else
+            scatter_planar_tile<VEC, MODE, G>(x, y, ysrc, idx, a, col, lds, waveBits, ib, rem);
     });
 }
 
@@ -534,7 +666,9 @@ __global__ __launch_bounds__(256) void k_copy_scalar(const float* __restrict__ s
 // Tile of the planar scatter.  16 KB tiles suit a launch that keeps every compute unit busy for several
 // rounds of workgroups; a launch of few workgroups finishes in one or two rounds, where the loads and the stores
 // of one round do not overlap much, and does better with 24 KB tiles (800x800x128 tensor, 27x27 blocks:
-// 9.08 -> 8.87 us at 58 blocks, 20.6 -> 19.9 us at 156, but 40.8 -> 41.4 us at 312).
+// 9.08 -> 8.87 us at 58 blocks, 20.6 -> 19.9 us at 156, but 40.8 -> 41.4 us at 312).  The 24 KB tile of that tensor
+// is moved in two halves (scatter_planar_tile_halves): 8.37 -> 7.64 us at 58 blocks, no change at 156; at 312 the
+// 16 KB tile stays ahead of it (38.5 against 40.0 us).
 constexpr int SCATTER_FEW_WGS_PER_CU = 22;
 
 // `share`: the launch does work for one block in `share` only (the passes of an overlapping add).
@@ -582,6 +716,13 @@ static bool launch_fixed_scatter(const float* x, float* y, const float* ysrc, co
     if constexpr (VEC == 4 && (MODE == SCATTER_ASSIGN || MODE == SCATTER_ADD || MODE == SCATTER_RANKED ||
                                MODE == SCATTER_RANKED_INLINE)) {
         // 27x27 blocks of 128 channels with 16 KB and 24 KB tiles; 16x16 blocks of 64 channels
+        if constexpr (MODE == SCATTER_ASSIGN || MODE == SCATTER_RANKED_INLINE) {
+            // (the 24 KB tile is what launches of few workgroups take: moved in two halves, see above)
+            if (y == ysrc &&
+                launch_fixed_scatter_one<VEC, MODE, TileFixedHalves<27, 27, 128, 184, 512>>(x, y, ysrc, idx, a, threads, lds,
+                                                                                             numActive, aux, stream))
+                return true;
+        }
         return launch_fixed_scatter_one<VEC, MODE, TileFixed<27, 27, 128, 124, 512>>(x, y, ysrc, idx, a, threads, lds,
                                                                                       numActive, aux, stream) ||
                launch_fixed_scatter_one<VEC, MODE, TileFixed<27, 27, 128, 184, 512>>(x, y, ysrc, idx, a, threads, lds,
