@@ -195,6 +195,11 @@ class Path:
         else:
             sc = M * sB + 2 * bin_s + 6 * M
         self.moved = {"reduce_mask": self.bytes["reduce_mask"], "gather": self.bytes["gather"], "scatter": sc}
+        # the gradient of the gather: as the reference composes it (zeros_like(x) written, then the atomic scatter-add
+        # reads the stack and reads and writes every covered element once per covering block); and what has to move
+        # (the stack read once, the tensor written once)
+        self.bytes["gather_backward"] = full + M * B + 2 * bin_g + 6 * M
+        self.moved["gather_backward"] = full + M * B + 6 * M
 
     def check(self, rc):
         if rc != 0:
@@ -278,13 +283,31 @@ class Path:
             out.append(e0.elapsed_time(e1) * 1e3 / reps)
         return statistics.median(out)
 
-    def op_table(self):
+    def gather_grad(self, i, M):
+        """The gradient of the gather with respect to x (sbnet_sparse_gather_grad): the stack scattered and summed
+        onto zeros; written into the set's `grad` tensor."""
+        s, wl = self.sets[i], self.wl
+        if "grad" not in s:
+            s["grad"] = self.torch.empty((self.N, self.H, self.W, self.C), dtype=self.torch.float32, device="cuda:0")
+            n = self.lib.sbnet_sparse_scatter_workspace_bytes(max(self.M, self.maxidx), self.dims, 4, self.bs, 2, self.bst, 2,
+                                                              self.bo, 2)
+            s["gws"] = self.torch.empty(max(n, 16), dtype=self.torch.uint8, device="cuda:0")
+        self.check(self.lib.sbnet_sparse_gather_grad(s["stack"].data_ptr(), M, s["idx"].data_ptr(), s["grad"].data_ptr(),
+                                                     self.dims, 4, self.bs, 2, self.bst, 2, self.bo, 2, int(wl.transpose),
+                                                     s["gws"].data_ptr(), s["gws"].numel(), self.stream))
+
+    def op_table(self, with_gather_grad=False):
         ops = {}
         if self.wl.mask is not None:
             ops["reduce_mask"] = self.time_op(lambda i: self.reduce(i, sync=False))
         if self.wl.x is not None:
             ops["gather"] = self.time_op(lambda i: self.gather(i, self.M))
         ops["scatter"] = self.time_op(lambda i: self.scatter(i, self.M))
+        if with_gather_grad and self.wl.x is not None:
+            ops["gather_backward"] = self.time_op(lambda i: self.gather_grad(i, self.M))
+            for s in self.sets:
+                s.pop("grad", None)
+                s.pop("gws", None)
         table = {}
         for k, us in ops.items():
             gbs, mgbs = self.bytes[k] / us * 1e-3, self.moved[k] / us * 1e-3
@@ -488,7 +511,7 @@ def main():
     path = None
     for d in densities:
         p = Path(workloads.config3(d), torch, lib, nsets=3)
-        table = p.op_table()
+        table = p.op_table(with_gather_grad=(d == args.density))
         table["M"] = p.M
         ops_by_density["%d%%" % round(d * 100)] = table
         if d == args.density:

@@ -185,6 +185,25 @@ int sbnet_sparse_gather_functor(const float* x, int N, int H, int W, int C, floa
                                 int numActive, const int16_t* activeBlockIndices, int transpose,
                                 void* stream);
 
+/* Gradient of sparse_gather with respect to x.  The reference registers it as a composition of its own ops,
+   sparse_scatter(grad, bin_counts, indices, zeros_like(x), ..., add=True, atomic=True, transpose)
+   (sparse_conv_lib.py:80-107, the same text in sbnet_ops/tests/test_sparse_blocks.py:36-62); this entry point computes
+   that tensor without materialising the zeros first:
+     dx = 0 everywhere, plus every block of dy at the block's place; where blocks overlap their values are summed.
+   dy is the block stack of the forward op's output layout ([num_active, R, S, C], or [num_active, C, R, S] with
+   transpose=1), dx a caller-allocated tensor of x's shape whose contents on entry do not matter.  With `workspace`
+   (sbnet_sparse_scatter_workspace_bytes() bytes for the same geometry) and at most 2x2 blocks over a pixel, zeros
+   are written only to the pixels that no block covers, and the blocks are added in ceil(R/U)*ceil(S/V) passes
+   of mutually non-overlapping blocks, each pixel's first value stored, later ones added: reproducible, equal to the
+   composition up to fp32 reassociation of at most four addends.  Otherwise dx is cleared and the atomic
+   scatter-add runs on it.  Checks and status codes as sbnet_sparse_scatter_var. */
+int sbnet_sparse_gather_grad(const float* dy, int32_t num_active, const int16_t* active_block_indices, float* dx,
+                             const int64_t* x_dims, int x_rank,
+                             const int32_t* bsize, int bsize_len,
+                             const int32_t* bstride, int bstride_len,
+                             const int32_t* boffset, int boffset_len,
+                             int transpose, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * sparse_scatter / sparse_scatter_var
  * ---------------------------------------------------------------------------------------- */

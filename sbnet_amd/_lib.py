@@ -44,6 +44,8 @@ SIGNATURES = {
     "sbnet_sparse_gather": (_int, [_vp, _i64p, _int, _i32, _vp, _i32p, _int, _i32p, _int, _i32p, _int, _int,
                                    _vp, _vp]),
     "sbnet_sparse_gather_functor": (_int, [_vp, _int, _int, _int, _int, _vp] + [_int] * 7 + [_vp, _int, _vp]),
+    "sbnet_sparse_gather_grad": (_int, [_vp, _i32, _vp, _vp, _i64p, _int, _i32p, _int, _i32p, _int, _i32p, _int, _int, _vp,
+                                        _sz, _vp]),
     "sbnet_sparse_scatter_workspace_bytes": (_sz, [_i32, _i64p, _int, _i32p, _int, _i32p, _int, _i32p, _int]),
     "sbnet_sparse_scatter": (_int, [_vp, _i32, _vp, _vp, _i64p, _int, _i32p, _int, _i32p, _int, _i32p, _int,
                                     _int, _int, _int, _vp, _vp, _sz, _vp]),

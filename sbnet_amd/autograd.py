@@ -5,7 +5,8 @@ The reference registers them in Python as compositions of its own ops
 sbnet_ops/tests/test_sparse_blocks.py:36-98); the same compositions are used here, so every
 backward pass runs the HIP kernels of the forward ops:
 
-* d SparseGather / dx       = sparse_scatter(grad, ..., zeros_like(x), add=True, atomic=True, transpose)
+* d SparseGather / dx       = sparse_scatter(grad, ..., zeros_like(x), add=True, atomic=True, transpose),
+                              computed by one entry point that writes zeros only where no block lies
 * d SparseScatter / dblocks = sparse_gather(grad, ...)
 * d SparseScatter / dybase  = grad                       (add=True)
                             = grad * stamp-out mask      (add=False; mask = blocks of zeros scattered over ones)
@@ -41,11 +42,9 @@ class SparseGatherFunction(torch.autograd.Function):
     def backward(ctx, grad):
         M, bsize, bstride, boffset, transpose = ctx.params
         (idx,) = ctx.saved_tensors
-        # the reference scatters onto zeros_like(x) with the copying op; adding in place onto fresh zeros
-        # gives the same tensor without the copy
-        dx = torch.zeros(ctx.x_shape, dtype=torch.float32, device=grad.device)
-        ops.scatter_forward(grad.contiguous(), [M], idx, dx, bsize, bstride, boffset, add=True, atomic=True,
-                            transpose=transpose, use_var=True)
+        # the reference scatters onto zeros_like(x) with the copying op; the library builds the same tensor without
+        # materialising the zeros first (sbnet_sparse_gather_grad)
+        dx = ops.gather_backward(grad.contiguous(), [M], idx, ctx.x_shape, bsize, bstride, boffset, transpose)
         return dx, None, None, None, None, None, None
 
 

@@ -554,6 +554,29 @@ int sbnet_sparse_scatter_var_device_count(const float* x, const int32_t* bin_cou
                           workspace, workspace_bytes, stream);
 }
 
+int sbnet_sparse_gather_grad(const float* dy, int32_t num_active, const int16_t* active_block_indices, float* dx,
+                             const int64_t* x_dims, int x_rank, const int32_t* bsize, int bsize_len,
+                             const int32_t* bstride, int bstride_len, const int32_t* boffset, int boffset_len,
+                             int transpose, void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (x_rank != 4) return SBNET_EINVAL_RANK;
+    if (!pair_ok(bsize, bsize_len) || !pair_ok(bstride, bstride_len) || !pair_ok(boffset, boffset_len))
+        return SBNET_EINVAL_PARAM_SHAPE;
+    if (!dx || !x_dims || !dims_fit_int(x_dims) || num_active < 0) return SBNET_EINVAL_ARG;
+    if (num_active > 0 && (!dy || !active_block_indices)) return SBNET_EINVAL_ARG;
+    if (!geom_ok((int)x_dims[0], (int)x_dims[1], (int)x_dims[2], (int)x_dims[3], bsize, bstride)) return SBNET_EINVAL_ARG;
+    const sbnet::Geom g = make_geom((int)x_dims[0], (int)x_dims[1], (int)x_dims[2], (int)x_dims[3], bsize, bstride, boffset);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    bool done = false;
+    SBNET_HIP(sbnet::launch_scatter_colored(dy, dx, active_block_indices, num_active, g, transpose != 0, workspace,
+                                            workspace_bytes, s, done, true));
+    if (done) return SBNET_OK;
+    // no scratch, or a geometry the passes do not take: zeros everywhere, then the atomic scatter-add
+    SBNET_HIP(sbnet::launch_zero(dx, (size_t)x_dims[0] * x_dims[1] * x_dims[2] * x_dims[3], s));
+    return scatter_impl(dy, num_active, nullptr, active_block_indices, dx, x_dims, bsize, bstride, boffset, 1, 1, transpose,
+                        workspace, workspace_bytes, s);
+}
+
 int sbnet_sparse_scatter_functor(const float* x, int N, int H, int W, int C, float* y, int bOffsH0,
                                  int bOffsW0, int bSzH, int bSzW, int bStrH, int bStrW, int numActive,
                                  const int16_t* activeBlockIndices, int add, int transpose, int atomic,

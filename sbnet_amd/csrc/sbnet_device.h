@@ -212,7 +212,34 @@ struct ColorArgs {
     const int32_t* dup;
     const int32_t* owner;  // SCATTER_OWNED: [N, H, W] list positions, -1 where no block covers the pixel
     const int32_t* rank;   // SCATTER_RANKED: nine bits per block, see k_rank_table
+    // SCATTER_COLOR with `first`: the passes add onto a tensor of which only the pixels that no block covers hold
+    // zeros yet (k_fill_uncovered), so a pass reads a pixel only where a block of an earlier pass has written it
+    // and stores 0 + v elsewhere.  `map` is the inverse block map [N, nBH, nBW] (list position or -1).
+    int first;
+    const int32_t* map;
+    int bhMin, bwMin, nBH, nBW;
+    // SCATTER_COLOR: the list sorted by pass (k_color_sort): perm[p * permStride + 0 .. counts[p]) are the list
+    // positions of pass p's blocks.  A pass then runs over its own blocks only, and the workgroups beyond them,
+    // which leave after one load, come last in the launch instead of in between (where each of them held up a
+    // working one).  NULL: every pass walks the whole list.
+    const int32_t* perm;
+    const int32_t* counts;
+    int permStride;
 };
+
+// Position `pos` of a colour pass's launch -> position in the block list, false when the pass has no such block.
+__device__ __forceinline__ bool color_block(const ColorArgs& col, uint32_t pos, uint32_t& ib)
+{
+    ib = pos;
+    if (!col.perm) return true;
+    typedef const int32_t __attribute__((address_space(4))) * const_i32_ptr;
+    // (two independent loads: the pass's count and the slot, which holds garbage beyond the count)
+    const int32_t cnt = *(const_i32_ptr)(reinterpret_cast<uintptr_t>(col.counts + col.pass));
+    const int32_t at = *(const_i32_ptr)(reinterpret_cast<uintptr_t>(col.perm + (int64_t)col.pass * col.permStride + pos));
+    if ((int32_t)pos >= cnt) return false;
+    ib = (uint32_t)at;
+    return true;
+}
 
 // Pixel (r, s) of a block against the block's nine bits: true when a block listed later covers it.
 __device__ __forceinline__ bool ranked_out(uint32_t bits, uint32_t r, uint32_t s, const Geom& g)
@@ -245,6 +272,38 @@ __device__ __forceinline__ uint32_t rank_bits(const ColorArgs& col, uint32_t ib)
 {
     typedef const int32_t __attribute__((address_space(4))) * const_i32_ptr;  // ib is wave-uniform: scalar load
     return (uint32_t)*(const_i32_ptr)(reinterpret_cast<uintptr_t>(col.rank + ib));
+}
+
+// SCATTER_COLOR with ColorArgs::first (at most 2x2 blocks over a pixel): nine bits like those of SCATTER_RANKED,
+// bit 3*rowClass + colClass set when an active block of an earlier pass covers that class of the block's pixels.
+// Eight look-ups in the inverse block map, all through the scalar unit (the block is the same for the workgroup).
+__device__ __forceinline__ uint32_t earlier_pass_bits(const ColorArgs& col, const BlockOrigin& o)
+{
+    typedef const int32_t __attribute__((address_space(4))) * const_i32_ptr;
+    // the eight neighbours' entries first (a neighbour beyond the map reads the block's own entry and is masked),
+    // then the arithmetic: eight independent scalar loads instead of a chain
+    int32_t other[9];
+    bool in[9];
+#pragma unroll
+    for (int q = 0; q < 9; ++q) {
+        const int dh = q / 3 - 1, dw = q % 3 - 1;
+        const int ih = o.bh + dh - col.bhMin, iw = o.bw + dw - col.bwMin;
+        in[q] = q != 4 && (unsigned)ih < (unsigned)col.nBH && (unsigned)iw < (unsigned)col.nBW;
+        const int64_t slot = ((int64_t)o.n * col.nBH + (in[q] ? ih : o.bh - col.bhMin)) * col.nBW + (in[q] ? iw : o.bw - col.bwMin);
+        other[q] = *(const_i32_ptr)(reinterpret_cast<uintptr_t>(col.map + slot));
+    }
+    uint32_t bits = 0u;
+#pragma unroll
+    for (int q = 0; q < 9; ++q) {
+        const int dh = q / 3 - 1, dw = q % 3 - 1;
+        // (kh and kw are 1 or 2 here: the pass of a block is the parity of its position)
+        const int pass = (((o.bh + dh) & (col.kh - 1)) * col.kw) + ((o.bw + dw) & (col.kw - 1));
+        if (in[q] && other[q] >= 0 && pass < col.pass) {
+            const uint32_t rows = dh < 0 ? 1u : (dh > 0 ? 4u : 7u), cols = dw < 0 ? 1u : (dw > 0 ? 4u : 7u);
+            bits |= ((rows & 1u) ? cols : 0u) | ((rows & 2u) ? cols << 3 : 0u) | ((rows & 4u) ? cols << 6 : 0u);
+        }
+    }
+    return bits;
 }
 
 // True when this launch has nothing to do for the block; `atomics` tells how to add otherwise.

@@ -65,9 +65,13 @@ hipError_t launch_scatter_pull(const float* x, float* y, const int16_t* idx, int
 // block positions per pass (either stack layout, up to 16 passes): reproducible, within rounding of the
 // sequential order.  Needs scratch of scatter_color_workspace_bytes(); `done` as above.
 size_t scatter_color_workspace_bytes(const Geom& g, int numActive);
+// ontoZeros: y is uninitialised and the result is zeros plus the blocks; the zeros are written by the call, and only
+// where no block covers a pixel when at most 2x2 blocks do (the passes then store a pixel's first value instead of
+// adding to it).
 hipError_t launch_scatter_colored(const float* x, float* y, const int16_t* idx, int numActive, const Geom& g,
                                   bool transpose, void* workspace, size_t workspaceBytes, hipStream_t stream,
-                                  bool& done);
+                                  bool& done, bool ontoZeros = false);
+hipError_t launch_zero(float* y, size_t count, hipStream_t stream);
 
 // Plain writes ("=") of overlapping blocks in the order of the sequential CPU functor: on a pixel that several
 // blocks cover, the block listed last wins (sparse_gather.cc:105-129), for either stack layout and for lists that

@@ -16,9 +16,10 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc_wide(const float* __restri
     uint32_t unit = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (unit >= a.units) return;
     unit = __builtin_amdgcn_readfirstlane(unit);
-    const uint32_t ib = fdiv(unit, a.dCpb);
-    if (beyond_count(a.g, ib)) return;
+    uint32_t ib = fdiv(unit, a.dCpb);
     const uint32_t chunk = unit - ib * a.cpb;
+    if (MODE == SCATTER_COLOR && !color_block(col, ib, ib)) return;
+    if (beyond_count(a.g, ib)) return;
     const BlockOrigin o = origin_of(load_triple(idx, ib), a.g);  // ib is wave-uniform: scalar load
     if (!o.valid) return;
     bool atomics = MODE == SCATTER_ATOMIC;
@@ -83,9 +84,10 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
     uint32_t unit = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (unit >= a.units) return;
     unit = __builtin_amdgcn_readfirstlane(unit);
-    const uint32_t ib = fdiv(unit, a.dCpb);
-    if (beyond_count(a.g, ib)) return;
+    uint32_t ib = fdiv(unit, a.dCpb);
     const uint32_t chunk = unit - ib * a.cpb;
+    if (MODE == SCATTER_COLOR && !color_block(col, ib, ib)) return;
+    if (beyond_count(a.g, ib)) return;
     const BlockOrigin o = origin_of(load_triple(idx, ib), a.g);
     if (!o.valid) return;
     bool atomics = MODE == SCATTER_ATOMIC;
@@ -129,8 +131,19 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
         for (int u = 0; u < NHWC_UNR; ++u) buf_store<BUF_NT>(yr, dst[u], v[u]);
     } else if (MODE == SCATTER_ADD || (MODE == SCATTER_COLOR && !atomics)) {
         vec cur[NHWC_UNR];
+        // (colour passes onto zeros: a pixel is read only where an earlier pass has written it; an out-of-range
+        // read returns 0, and 0 + v is what a pixel's first write stores)
+        const uint32_t ebits = MODE == SCATTER_COLOR && col.first ? earlier_pass_bits(col, o) : 0x1ffu;
 #pragma unroll
-        for (int u = 0; u < NHWC_UNR; ++u) cur[u] = buf_load<VEC>(sr, dst[u]);
+        for (int u = 0; u < NHWC_UNR; ++u) {
+            uint32_t src = dst[u];
+            if (MODE == SCATTER_COLOR && col.first) {
+                const uint32_t e = e0 + u * 64;
+                const uint32_t r = fdiv(e, a.dRow);
+                if (!ranked_out(ebits, r, fdiv(e - r * a.rowV, a.dCV), a.g)) src = BUF_OOB;
+            }
+            cur[u] = buf_load<VEC>(sr, src);
+        }
 #pragma unroll
         for (int u = 0; u < NHWC_UNR; ++u) buf_store<BUF_NT>(yr, dst[u], vadd(cur[u], v[u]));
     } else {
@@ -156,6 +169,7 @@ __device__ __forceinline__ void scatter_planar_tile(const float* __restrict__ x,
     const uint32_t tid = threadIdx.x, nthr = G::nthr(a);
     const uint32_t RS = G::RS(a), Pp = G::Pp(a), vpr = G::vpr(a);
     TileId t;
+    if (MODE == SCATTER_COLOR && !color_block(col, ib, ib)) return;
     decode_tile<G>(a, t, ib, rem);
     const RawTriple raw = load_triple(idx, t.ib);  // scalar load, needed only after the barrier
     if (beyond_count(a.g, t.ib)) return;
@@ -220,6 +234,8 @@ __device__ __forceinline__ void scatter_planar_tile(const float* __restrict__ x,
         fetch_rows();
     }
     const BlockOrigin o = origin_of(raw, a.g);
+    // (colour passes onto zeros: the neighbours' map entries, fetched while the tile's loads are in flight)
+    const uint32_t ebits = MODE == SCATTER_COLOR && col.first && o.valid ? earlier_pass_bits(col, o) : 0x1ffu;
     if (MODE == SCATTER_RANKED_INLINE) {
         // nine bits: classes of this block's pixels that a block listed later covers (the later one wins them)
         uint32_t bits = 0u;
@@ -240,36 +256,58 @@ __device__ __forceinline__ void scatter_planar_tile(const float* __restrict__ x,
             for (int off = 32; off > 0; off >>= 1) bits |= (uint32_t)__shfl_xor((int)bits, off);
         if ((tid & 63u) == 0u) waveBits[tid >> 6] = bits;
     }
-    lds_barrier();
+    if (!o.valid) return;  // (the whole workgroup)
 
     // NHWC side: LDS -> base tensor; pixels outside the image are dropped (sparse_gather.cc:121)
-    if (!o.valid) return;
     float* img = y + (int64_t)o.n * a.imgFloats;
     const rsrc_t yr = make_rsrc(img, a.imgBytes);
     const rsrc_t sr = make_rsrc(ysrc + (int64_t)o.n * a.imgFloats, a.imgBytes);  // what an add reads
     const uint32_t c0l = (tid & ((1u << G::lppLog(a)) - 1u)) * VEC;
-    vec w[TILE_LD];
-    uint32_t offs[TILE_LD];
+    vec w[TILE_LD], cur[TILE_LD];
+    uint32_t offs[TILE_LD], pls[TILE_LD];
     int32_t own[TILE_LD];
     const rsrc_t wr = make_rsrc(MODE == SCATTER_OWNED ? col.owner + (int64_t)o.n * a.g.H * a.g.W : nullptr,
                                 MODE == SCATTER_OWNED ? (uint32_t)(a.g.H * a.g.W) * 4u : 0u);
     uint32_t rbits = MODE == SCATTER_RANKED ? rank_bits(col, t.ib) : 0u;
-    if (MODE == SCATTER_RANKED_INLINE) {
-        for (uint32_t w = 0; w < (nthr >> 6); ++w) rbits |= waveBits[w];
+    // colour passes onto zeros: a pixel is read only where a block of an earlier pass has written it (an out-of-range
+    // read returns 0, and 0 + v is what a pixel's first write stores)
+    bool rmw[TILE_LD];
+    auto walk = [&]() {
+        nhwc_walk<VEC, G>(a, t, o, tid, nthr, [&](int u, uint32_t pl, uint32_t off, uint32_t pix, uint32_t r, uint32_t sc) {
+            if ((MODE == SCATTER_RANKED || MODE == SCATTER_RANKED_INLINE) && ranked_out(rbits, r, sc, a.g)) off = BUF_OOB;
+            rmw[u] = MODE != SCATTER_COLOR || ranked_out(ebits, r, sc, a.g);
+            offs[u] = off;
+            pls[u] = pl;
+            if (MODE == SCATTER_OWNED) own[u] = __builtin_bit_cast(int32_t, buf_load<1>(wr, off != BUF_OOB ? pix * 4u : BUF_OOB));
+        });
+    };
+    // An add's reads of the base do not depend on the tile: they go out before the barrier, behind the tile's loads.
+    constexpr bool EARLY = MODE == SCATTER_ADD || MODE == SCATTER_COLOR;
+    if (EARLY) {
+        walk();
+        if (!atomics) {
+#pragma unroll
+            for (int u = 0; u < TILE_LD; ++u) cur[u] = buf_load<VEC>(sr, MODE == SCATTER_COLOR && !rmw[u] ? BUF_OOB : offs[u]);
+        }
     }
-    nhwc_walk<VEC, G>(a, t, o, tid, nthr, [&](int u, uint32_t pl, uint32_t off, uint32_t pix, uint32_t r, uint32_t sc) {
-        if ((MODE == SCATTER_RANKED || MODE == SCATTER_RANKED_INLINE) && ranked_out(rbits, r, sc, a.g)) off = BUF_OOB;
-        offs[u] = off;
-        if (MODE == SCATTER_OWNED) own[u] = __builtin_bit_cast(int32_t, buf_load<1>(wr, off != BUF_OOB ? pix * 4u : BUF_OOB));
+    lds_barrier();
+    if (!EARLY) {
+        if (MODE == SCATTER_RANKED_INLINE) {
+            for (uint32_t wv = 0; wv < (nthr >> 6); ++wv) rbits |= waveBits[wv];
+        }
+        walk();
+    }
+#pragma unroll
+    for (int u = 0; u < TILE_LD; ++u) {
         w[u] = vzero<VEC>();
-        if (off != BUF_OOB) {
+        if (offs[u] != BUF_OOB) {
 #pragma unroll
             for (int k = 0; k < VEC; ++k) {
                 const uint32_t c = c0l + k;
-                vset(w[u], k, lds[c * Pp + (pl ^ lds_swz(c))]);
+                vset(w[u], k, lds[c * Pp + (pls[u] ^ lds_swz(c))]);
             }
         }
-    });
+    }
     if (MODE == SCATTER_OWNED) {
 #pragma unroll
         for (int u = 0; u < TILE_LD; ++u) buf_store<BUF_NT>(yr, own[u] == (int32_t)t.ib ? offs[u] : BUF_OOB, w[u]);
@@ -277,9 +315,6 @@ __device__ __forceinline__ void scatter_planar_tile(const float* __restrict__ x,
 #pragma unroll
         for (int u = 0; u < TILE_LD; ++u) buf_store<BUF_NT>(yr, offs[u], w[u]);
     } else if (MODE == SCATTER_ADD || (MODE == SCATTER_COLOR && !atomics)) {
-        vec cur[TILE_LD];
-#pragma unroll
-        for (int u = 0; u < TILE_LD; ++u) cur[u] = buf_load<VEC>(sr, offs[u]);
 #pragma unroll
         for (int u = 0; u < TILE_LD; ++u) buf_store<BUF_NT>(yr, offs[u], vadd(cur[u], w[u]));
     } else {
@@ -455,6 +490,7 @@ __global__ __launch_bounds__(512) void k_scatter_planar(const float* __restrict_
 // be represented in the map; k_pull_map notices, and k_scatter_pull then falls back to hardware atomics
 // for the whole launch (still correct, to rounding).
 
+constexpr int STRIP_ROWS = 4;    // image rows per workgroup of the kernels that walk the output in row order
 constexpr int PULL_STEPS = 3;    // 64-vector steps of one wave, all in flight together (1: 223 us, 2: 228, 3: 211, 4: 232
                                  // on the 16x16-at-stride-8, 256-channel workload; 5 and more run out of registers)
 constexpr int PULL_CLASSES = 9;  // 3 row classes x 3 column classes of a block's pixels (see below)
@@ -714,7 +750,7 @@ static bool launch_fixed_scatter(const float* x, float* y, const float* ysrc, co
                                  int threads, size_t lds, int numActive, const ColorArgs& aux, hipStream_t stream)
 {
     if constexpr (VEC == 4 && (MODE == SCATTER_ASSIGN || MODE == SCATTER_ADD || MODE == SCATTER_RANKED ||
-                               MODE == SCATTER_RANKED_INLINE)) {
+                               MODE == SCATTER_RANKED_INLINE || MODE == SCATTER_COLOR)) {
         // 27x27 blocks of 128 channels with 16 KB and 24 KB tiles; 16x16 blocks of 64 channels
         if constexpr (MODE == SCATTER_ASSIGN || MODE == SCATTER_RANKED_INLINE) {
             // (the 24 KB tile is what launches of few workgroups take: moved in two halves, see above)
@@ -766,7 +802,7 @@ static void scatter_dispatch(const float* x, float* y, const float* ysrc, const 
 {
     // `order`: the owner map (SCATTER_OWNED) or the rank table (SCATTER_RANKED)
     const ColorArgs aux{1, 1, 0, nullptr, MODE == SCATTER_OWNED ? order : nullptr,
-                        MODE == SCATTER_RANKED ? order : nullptr};
+                        MODE == SCATTER_RANKED ? order : nullptr, 0, nullptr, 0, 0, 0, 0, nullptr, nullptr, 0};
     const int32_t* owner = order;
     if (!transpose) {
         NhwcArgs a;
@@ -921,6 +957,35 @@ hipError_t launch_scatter_pull(const float* x, float* y, const int16_t* idx, int
 // ---- scatter-add in passes ------------------------------------------------------------------
 
 constexpr int COLOR_MAX_PASSES = 16;
+constexpr int COLOR_SORT_MAX_BLOCKS = 1 << 17;  // lists that one workgroup sorts by pass in a few microseconds
+
+// The list sorted by colour pass (see ColorArgs::perm).  One workgroup: counts per pass, offsets, then every row's
+// position goes to the next free slot of its pass (the order inside a pass does not matter: its blocks do not
+// overlap).  When the list names a block twice the passes fall back to hardware atomics, all in pass 0.
+__global__ __launch_bounds__(1024) void k_color_sort(const int16_t* __restrict__ idx, int numActive, Geom g, int kh, int kw,
+                                                     const int32_t* __restrict__ dup, int32_t* __restrict__ counts,
+                                                     int32_t* __restrict__ perm, int permStride)
+{
+    __shared__ int next[COLOR_MAX_PASSES];
+    const int tid = (int)threadIdx.x;
+    int count = numActive;
+    if (g.countDev) count = min(count, max(*g.countDev, 0));
+    const bool all0 = *dup != 0;
+    if (tid < COLOR_MAX_PASSES) next[tid] = 0;
+    __syncthreads();
+    for (int i = tid; i < count; i += 1024) {
+        int p = 0;
+        if (!all0) {
+            int mh = idx[(size_t)i * 3 + 1] % kh, mw = idx[(size_t)i * 3 + 2] % kw;
+            if (mh < 0) mh += kh;
+            if (mw < 0) mw += kw;
+            p = mh * kw + mw;
+        }
+        perm[(int64_t)p * permStride + atomicAdd(&next[p], 1)] = i;
+    }
+    __syncthreads();
+    if (tid < COLOR_MAX_PASSES) counts[tid] = next[tid];
+}
 
 size_t scatter_color_workspace_bytes(const Geom& g, int numActive)
 {
@@ -928,7 +993,9 @@ size_t scatter_color_workspace_bytes(const Geom& g, int numActive)
     int64_t mapN = 0;
     const int64_t Kh = ((int64_t)g.R + g.U - 1) / g.U, Kw = ((int64_t)g.S + g.V - 1) / g.V;
     if (numActive <= 0 || Kh * Kw > COLOR_MAX_PASSES || !make_map_args(g, a, mapN)) return 0;
-    return (size_t)mapN * 4 + 16;
+    // the block map, the duplicate flag, the passes' counts, one list of the capacity of the whole list per pass
+    const size_t perm = numActive <= COLOR_SORT_MAX_BLOCKS ? (size_t)numActive * (size_t)(Kh * Kw) * 4 : 0;
+    return (size_t)mapN * 4 + 16 + COLOR_MAX_PASSES * 4 + perm;
 }
 
 template <int VEC>
@@ -953,19 +1020,151 @@ static bool color_passes(const float* x, float* y, const int16_t* idx, const Geo
         size_t lds;
         unsigned grid;
         if ((int64_t)g.R * g.S < 4 || !scatter_tile_args(g, numActive, VEC, a, threads, lds, grid, passes)) return false;
-        for (col.pass = 0; col.pass < passes; ++col.pass)
+        for (col.pass = 0; col.pass < passes; ++col.pass) {
+            if (launch_fixed_scatter<VEC, SCATTER_COLOR>(x, y, y, idx, a, threads, lds, numActive, col, stream)) continue;
             hipLaunchKernelGGL((k_scatter_planar<VEC, SCATTER_COLOR, TileRt>), tile_grid(a.grid2d, a.tpb, numActive, a.total, a.g),
                                dim3(threads), lds, stream, x, y, (const float*)y, idx, a, col);
+        }
     }
     return true;
 }
 
+// ---- zero-filling for "scatter-add onto zeros" (the gradient of sparse_gather) ------------------------------
+
+__global__ __launch_bounds__(256) void k_fill_zero(f4* __restrict__ y, size_t n4, float* __restrict__ tail, int nTail)
+{
+    const size_t base = (size_t)blockIdx.x * (256 * COPY_UNR) + threadIdx.x;
+#pragma unroll
+    for (int u = 0; u < COPY_UNR; ++u) {
+        const size_t i = base + (size_t)u * 256;
+        if (i < n4) st_stream(y + i, (f4)(0.f));
+    }
+    if (blockIdx.x == 0 && (int)threadIdx.x < nTail) tail[threadIdx.x] = 0.f;
+}
+
+static void launch_fill_zero(float* y, size_t count, hipStream_t stream)
+{
+    // (16-byte stores from the first aligned float on; the few floats before and after it one by one)
+    const uintptr_t p = reinterpret_cast<uintptr_t>(y);
+    size_t head = ((16 - (p & 15)) & 15) / 4;
+    if (head > count) head = count;
+    const size_t n4 = (count - head) / 4, rest = count - head - n4 * 4;
+    const size_t per = 256 * COPY_UNR;
+    if (n4) hipLaunchKernelGGL(k_fill_zero, dim3((unsigned)((n4 + per - 1) / per)), dim3(256), 0, stream,
+                               reinterpret_cast<f4*>(y + head), n4, y + head + n4 * 4, (int)rest);
+    else if (rest) hipLaunchKernelGGL(k_fill_zero, dim3(1), dim3(256), 0, stream, reinterpret_cast<f4*>(y + head), (size_t)0,
+                                      y + head, (int)rest);
+    if (head) hipLaunchKernelGGL(k_fill_zero, dim3(1), dim3(256), 0, stream, reinterpret_cast<f4*>(y), (size_t)0, y, (int)head);
+}
+
+// Zeros for the pixels that no active block covers (at most 2x2 blocks over a pixel); the colour passes that follow
+// write every covered pixel themselves (ColorArgs::first).  Strips of 4 image rows of one row of stride cells, 256
+// channel vectors wide, as in k_scatter_strip; a pixel of cell (bh, bw) can be covered by the blocks (bh, bw),
+// (bh, bw-1), (bh-1, bw) and (bh-1, bw-1).  When the list names a block twice the passes fall back to hardware
+// atomics, which need zeros everywhere: then every pixel is cleared.
+struct FillArgs {
+    Geom g;
+    int bhMin, bwMin, nBH, nBW;  // extent of the inverse block map
+    int cellH0, cellW0;          // first row / column of stride cells that touches the image
+    int nBands;                  // rows of cells that touch the image
+    uint32_t kPerBand, CV, PX, nPC, imgBytes;
+    int64_t imgFloats;
+    FastDiv dCV, dV, dK, dPC, dBands;
+};
+
+__device__ __forceinline__ bool fill_block_active(const FillArgs& a, const int32_t* __restrict__ map, uint32_t n, int bh,
+                                                  int bw)
+{
+    const int ih = bh - a.bhMin, iw = bw - a.bwMin;
+    if ((unsigned)ih >= (unsigned)a.nBH || (unsigned)iw >= (unsigned)a.nBW) return false;
+    return map[((int64_t)n * a.nBH + ih) * a.nBW + iw] >= 0;
+}
+
+template <int VEC>
+__global__ __launch_bounds__(256) void k_fill_uncovered(float* __restrict__ y, const int32_t* __restrict__ map,
+                                                        const int32_t* __restrict__ dup, FillArgs a)
+{
+    typedef const int32_t __attribute__((address_space(4))) * const_i32_ptr;
+    const uint32_t tid = threadIdx.x;
+    uint32_t l = blockIdx.x;
+    uint32_t t = fdiv(l, a.dPC);
+    const uint32_t pc = (uint32_t)__builtin_amdgcn_readfirstlane((int)(l - t * a.nPC));
+    l = t; t = fdiv(l, a.dK);
+    const int r0 = __builtin_amdgcn_readfirstlane((int)(l - t * a.kPerBand)) * STRIP_ROWS;
+    l = t; t = fdiv(l, a.dBands);
+    const int bh = __builtin_amdgcn_readfirstlane((int)(l - t * (uint32_t)a.nBands)) + a.cellH0;
+    const uint32_t n = (uint32_t)__builtin_amdgcn_readfirstlane((int)t);
+    const int hTop = a.g.oh + bh * a.g.U + r0;
+
+    const uint32_t wl = fdiv(tid, a.dCV), cv = tid - wl * a.CV;
+    const uint32_t w = pc * a.PX + wl;
+    const bool live = wl < a.PX && w < (uint32_t)a.g.W;
+    const uint32_t dw = w - (uint32_t)(a.g.ow + a.cellW0 * a.g.V);
+    const uint32_t iw = fdiv(dw, a.dV);
+    const int sc = (int)(dw - iw * (uint32_t)a.g.V), bw = (int)iw + a.cellW0;
+
+    const bool all = *(const_i32_ptr)(reinterpret_cast<uintptr_t>(dup)) != 0;
+    // the block of the pixel's own cell and of the cell to its left, in this row of cells and in the one above
+    const bool left = sc + a.g.V < a.g.S, here = sc < a.g.S;
+    bool cur = false, up = false;
+    if (live && !all) {
+        cur = (here && fill_block_active(a, map, n, bh, bw)) || (left && fill_block_active(a, map, n, bh, bw - 1));
+        if (r0 + a.g.U < a.g.R)  // (some row of the strip lies under the blocks of the row of cells above)
+            up = (here && fill_block_active(a, map, n, bh - 1, bw)) || (left && fill_block_active(a, map, n, bh - 1, bw - 1));
+    }
+    const rsrc_t yr = make_rsrc(y + (int64_t)n * a.imgFloats, a.imgBytes);
+#pragma unroll
+    for (int u = 0; u < STRIP_ROWS; ++u) {
+        const int r = r0 + u, h = hTop + u;
+        const bool covered = (cur && r < a.g.R) || (up && r + a.g.U < a.g.R);
+        const bool write = live && r < a.g.U && (unsigned)h < (unsigned)a.g.H && !covered;
+        buf_store<BUF_NT>(yr, write ? (((uint32_t)h * (uint32_t)a.g.W + w) * a.CV + cv) * (uint32_t)(VEC * 4) : BUF_OOB,
+                          vzero<VEC>());
+    }
+}
+
+static bool make_fill_args(const Geom& g, int vec, const PullArgs& pa, FillArgs& a, unsigned& grid)
+{
+    if (g.R > 2 * (int64_t)g.U || g.S > 2 * (int64_t)g.V) return false;  // at most 2x2 blocks over a pixel
+    a.g = g;
+    a.imgFloats = (int64_t)g.H * g.W * g.C;
+    if (a.imgFloats >= (1ll << 30)) return false;
+    a.imgBytes = (uint32_t)(a.imgFloats * 4);
+    a.bhMin = pa.bhMin; a.bwMin = pa.bwMin; a.nBH = pa.nBH; a.nBW = pa.nBW;
+    auto floordiv = [](int64_t p, int64_t q) { return p >= 0 ? p / q : -((-p + q - 1) / q); };
+    const int64_t h0 = floordiv(-(int64_t)g.oh, g.U), h1 = floordiv((int64_t)g.H - 1 - g.oh, g.U);
+    const int64_t w0 = floordiv(-(int64_t)g.ow, g.V);
+    if (h0 < -(1ll << 30) || h1 > (1ll << 30) || w0 < -(1ll << 30) || w0 > (1ll << 30)) return false;
+    a.cellH0 = (int)h0; a.cellW0 = (int)w0;
+    a.nBands = (int)(h1 - h0 + 1);
+    a.kPerBand = (uint32_t)((g.U + STRIP_ROWS - 1) / STRIP_ROWS);
+    a.CV = (uint32_t)(g.C / vec);
+    if (a.CV > 256u) return false;
+    a.PX = 256u / a.CV;
+    a.nPC = ((uint32_t)g.W + a.PX - 1u) / a.PX;
+    const int64_t tiles = (int64_t)g.N * a.nBands * a.kPerBand * a.nPC;
+    if (tiles >= (1ll << 31)) return false;
+    grid = (unsigned)tiles;
+    a.dCV = make_fastdiv(a.CV);
+    a.dV = make_fastdiv((uint32_t)g.V);
+    a.dK = make_fastdiv(a.kPerBand);
+    a.dPC = make_fastdiv(a.nPC);
+    a.dBands = make_fastdiv((uint32_t)a.nBands);
+    return true;
+}
+
+// ontoZeros: y holds nothing yet and the result is "zeros, plus the blocks" (the gradient of sparse_gather,
+// sparse_conv_lib.py:80-107): the zeros are written here, only where they are needed when the geometry allows.
 hipError_t launch_scatter_colored(const float* x, float* y, const int16_t* idx, int numActive, const Geom& g,
                                   bool transpose, void* workspace, size_t workspaceBytes, hipStream_t stream,
-                                  bool& done)
+                                  bool& done, bool ontoZeros)
 {
     done = false;
-    if (numActive == 0) { done = true; return hipSuccess; }
+    if (numActive == 0) {
+        if (ontoZeros) launch_fill_zero(y, (size_t)g.N * g.H * g.W * g.C, stream);
+        done = true;
+        return hipGetLastError();
+    }
     const size_t need = scatter_color_workspace_bytes(g, numActive);
     if (!workspace || need == 0 || workspaceBytes < need || (reinterpret_cast<uintptr_t>(workspace) & 3))
         return hipSuccess;
@@ -976,9 +1175,20 @@ hipError_t launch_scatter_colored(const float* x, float* y, const int16_t* idx, 
     col.kh = (g.R + g.U - 1) / g.U;
     col.kw = (g.S + g.V - 1) / g.V;
     col.pass = 0;
+    col.owner = nullptr;
+    col.rank = nullptr;
     int32_t* map = static_cast<int32_t*>(workspace);
     int32_t* dup = map + mapN;
     col.dup = dup;
+    col.first = 0;
+    col.map = map;
+    col.bhMin = pa.bhMin; col.bwMin = pa.bwMin; col.nBH = pa.nBH; col.nBW = pa.nBW;
+    int32_t* counts = dup + 4;
+    int32_t* perm = counts + COLOR_MAX_PASSES;
+    const bool sorted = numActive <= COLOR_SORT_MAX_BLOCKS && col.kh * col.kw > 1;
+    col.perm = sorted ? perm : nullptr;
+    col.counts = sorted ? counts : nullptr;
+    col.permStride = numActive;
     // geometry checks first: nothing is launched unless the passes can run
     const int vec = pick_vec(g, y, transpose ? nullptr : x);
     {
@@ -991,17 +1201,41 @@ hipError_t launch_scatter_colored(const float* x, float* y, const int16_t* idx, 
                        : ((int64_t)g.R * g.S < 4 || !scatter_tile_args(g, numActive, vec, ta, threads, lds, grid, col.kh * col.kw)))
             return hipSuccess;
     }
+    FillArgs fa;
+    unsigned fillGrid = 0;
+    // (the kernels that read only what an earlier pass wrote are the buffer-addressed ones)
+    const bool partial = ontoZeros && (transpose || nhwc_fits_buffers(g)) && make_fill_args(g, vec, pa, fa, fillGrid);
     int64_t fillWgs = (mapN + 255) / 256;
     if (fillWgs > 4096) fillWgs = 4096;
     if (fillWgs < 1) fillWgs = 1;
     hipLaunchKernelGGL(k_pull_fill, dim3((unsigned)fillWgs), dim3(256), 0, stream, map, mapN, dup);
     hipLaunchKernelGGL(k_pull_map, dim3((unsigned)((numActive + 255) / 256)), dim3(256), 0, stream, idx, numActive, pa,
                        map, dup);
+    if (sorted)
+        hipLaunchKernelGGL(k_color_sort, dim3(1), dim3(1024), 0, stream, idx, numActive, g, col.kh, col.kw,
+                           (const int32_t*)dup, counts, perm, numActive);
+    if (partial) {
+        col.first = 1;
+        const int32_t* cmap = map;
+        const int32_t* cdup = dup;
+        if (vec == 4) hipLaunchKernelGGL(k_fill_uncovered<4>, dim3(fillGrid), dim3(256), 0, stream, y, cmap, cdup, fa);
+        else if (vec == 2) hipLaunchKernelGGL(k_fill_uncovered<2>, dim3(fillGrid), dim3(256), 0, stream, y, cmap, cdup, fa);
+        else hipLaunchKernelGGL(k_fill_uncovered<1>, dim3(fillGrid), dim3(256), 0, stream, y, cmap, cdup, fa);
+    } else if (ontoZeros) {
+        launch_fill_zero(y, (size_t)g.N * g.H * g.W * g.C, stream);
+    }
     const int passes = col.kh * col.kw;
     if (vec == 4) color_passes<4>(x, y, idx, g, numActive, transpose, col, passes, stream);
     else if (vec == 2) color_passes<2>(x, y, idx, g, numActive, transpose, col, passes, stream);
     else color_passes<1>(x, y, idx, g, numActive, transpose, col, passes, stream);
     done = true;
+    return hipGetLastError();
+}
+
+// Fills y with zeros (for callers of the zero-based scatter-add that take another path).
+hipError_t launch_zero(float* y, size_t count, hipStream_t stream)
+{
+    launch_fill_zero(y, count, stream);
     return hipGetLastError();
 }
 
@@ -1042,7 +1276,6 @@ struct StripArgs {
     FastDiv dCVT, dV, dK, dCC, dPC, dBH, dS4, dCT;
 };
 
-constexpr int STRIP_ROWS = 4;
 
 // Cell of block (n, bh, bw) in the map, or -1 when the block cannot touch the image.
 __device__ __forceinline__ int64_t cell_slot(const StripArgs& a, int n, int bh, int bw)

@@ -250,6 +250,36 @@ def gather_forward(x, bin_counts, active_block_indices, dynamic_bsize, dynamic_b
     return y
 
 
+def gather_backward(grad, bin_counts, active_block_indices, x_shape, dynamic_bsize, dynamic_bstride, dynamic_boffset,
+                    transpose=False):
+    """Gradient of sparse_gather with respect to x (sparse_conv_lib.py:80-107: the reference scatters grad onto
+    zeros_like(x) with add=True, atomic=True): a tensor of shape x_shape that is zero where no block lies and holds
+    the sum of the blocks of `grad` elsewhere, built without clearing the tensor first."""
+    lib = _lib.load()
+    grad = _dev_f32(grad, "grad")
+    idx = _idx_i16(active_block_indices)
+    M = _count(bin_counts)
+    bs, bsp, bsl = _pair(dynamic_bsize)
+    bt, btp, btl = _pair(dynamic_bstride)
+    bo, bop, bol = _pair(dynamic_boffset)
+    x_shape = tuple(int(d) for d in x_shape)
+    dims = (ctypes.c_int64 * max(len(x_shape), 4))(*(list(x_shape) + [1] * max(0, 4 - len(x_shape))))
+    rank = len(x_shape)
+    if rank == 4 and bsl == 2 and btl == 2 and bol == 2:
+        _check_count(M, idx)
+        _check_stack(grad, M, x_shape[3], int(bs[0]), int(bs[1]), transpose, "grad")
+    with torch.cuda.device(grad.device):
+        dx = torch.empty(x_shape, dtype=torch.float32, device=grad.device)
+        ws_ptr, ws_bytes = None, 0
+        need = lib.sbnet_sparse_scatter_workspace_bytes(M, dims, rank, bsp, bsl, btp, btl, bop, bol)
+        if need:
+            ws = _workspace(grad.device, need)
+            ws_ptr, ws_bytes = ws.data_ptr(), ws.numel()
+        _check(lib.sbnet_sparse_gather_grad(grad.data_ptr(), M, idx.data_ptr(), dx.data_ptr(), dims, rank, bsp, bsl, btp,
+                                            btl, bop, bol, int(bool(transpose)), ws_ptr, ws_bytes, _stream()))
+    return dx
+
+
 def scatter_forward(x, bin_counts, active_block_indices, ybase, dynamic_bsize, dynamic_bstride, dynamic_boffset, add,
                     atomic, transpose, use_var, scratch=True):
     """The scatter without autograd bookkeeping.  scratch=False passes no workspace to the library (hardware

@@ -181,6 +181,43 @@ def test_scatter_backward_matches_oracle(case, add, transpose):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("case", [
+    # (N, H, W, C), bsize, bstride, boffset, repeated rows
+    ((2, 64, 72, 32), (10, 10), (8, 8), (-1, -1), False),      # 2x2 blocks over a pixel: zeros only where no block lies
+    ((1, 120, 130, 128), (27, 27), (25, 25), (-1, -1), False),  # planes split over tiles, four channel chunks
+    ((2, 50, 61, 24), (7, 9), (5, 6), (2, -4), False),         # uneven everything, 6 channel vectors per pixel
+    ((3, 33, 47, 5), (5, 7), (3, 4), (-2, -3), False),         # scalar channel vectors
+    ((2, 40, 44, 16), (4, 4), (6, 7), (1, 0), False),          # gaps: one pass
+    ((1, 30, 30, 8), (7, 7), (2, 2), (0, 0), False),           # 4x4 blocks over a pixel: cleared first, 16 passes
+    ((2, 64, 72, 32), (10, 10), (8, 8), (-1, -1), True),       # a list that names blocks twice: hardware atomics
+    ((1, 20, 20, 4), (1, 3), (1, 2), (0, 0), False),           # planes below 4 pixels
+], ids=lambda c: "x".join(map(str, c[0])) + "_b%dx%d_s%dx%d%s" % (c[1] + c[2] + ("_dups" if c[4] else "",)))
+def test_gather_grad_entry_point(case):
+    """sbnet_sparse_gather_grad (through ops.gather_backward) against the oracle's composition
+    scatter(grad, zeros, add, atomic) on shuffled lists, into a tensor that holds garbage on entry."""
+    from sbnet_amd import ops
+    shape, bs, bst, bo, dups = case
+    rng, idx, cnt = setup_case(case[:4], 23)
+    if dups:
+        idx = np.concatenate([idx, idx[:4]])
+    rng.shuffle(idx, axis=0)
+    cnt = np.array([len(idx)], np.int32)
+    M, C = len(idx), shape[3]
+    for transpose in (False, True):
+        gshape = (M, C, bs[0], bs[1]) if transpose else (M, bs[0], bs[1], C)
+        g = rng.integers(-8, 9, size=gshape).astype(np.float32)
+        exp = orc.sparse_gather_grad(g, shape, cnt, idx, bs, bst, bo, transpose=transpose)
+        for rep in range(2):   # (the second call finds the first one's values in the allocator's memory)
+            dx = ops.gather_backward(dev(g), cnt, dev(idx), shape, bs, bst, bo, transpose)
+            np.testing.assert_array_equal(dx.cpu().numpy(), exp, err_msg="transpose %s" % transpose)
+            del dx
+        # fewer rows than the list holds
+        exp2 = orc.sparse_gather_grad(g, shape, [M - 2], idx, bs, bst, bo, transpose=transpose)
+        dx = ops.gather_backward(dev(g), [M - 2], dev(idx), shape, bs, bst, bo, transpose)
+        np.testing.assert_array_equal(dx.cpu().numpy(), exp2)
+
+
+@pytest.mark.gpu
 def test_chain_gather_multiply_scatter_backward():
     """x -> gather -> * w -> scatter(add) onto ybase -> sum(. * v): gradients through both Functions at once,
     against the chain rule spelled out with the oracle's pieces."""
