@@ -546,7 +546,8 @@ static bool launch_fixed_lines(const float* x, float* y, const int16_t* idx, con
     // 27x27 blocks of 128 channels (800x800x128 tensor): three and two splits per plane; 18x18 blocks of 64 channels
     return launch_fixed_lines_one<LinesFixed<27, 27, 128, 3, 512>>(x, y, idx, a, threads, ld, lds, numActive, stream) ||
            launch_fixed_lines_one<LinesFixed<27, 27, 128, 2, 512>>(x, y, idx, a, threads, ld, lds, numActive, stream) ||
-           launch_fixed_lines_one<LinesFixed<18, 18, 64, 2, 512>>(x, y, idx, a, threads, ld, lds, numActive, stream);
+           launch_fixed_lines_one<LinesFixed<18, 18, 64, 2, 512>>(x, y, idx, a, threads, ld, lds, numActive, stream) ||
+           launch_fixed_lines_one<LinesFixed<18, 18, 256, 2, 512>>(x, y, idx, a, threads, ld, lds, numActive, stream);
 }
 
 template <int VEC>
@@ -617,7 +618,8 @@ int tile_choice(int kind, const Geom& g, int numActive, int vec, int yAlignedTo,
         out[9] = RS - (a.psplit - 1) * a.P;
         out[10] = lines_match<LinesFixed<27, 27, 128, 3, 512>>(a, threads, ld) ||
                   lines_match<LinesFixed<27, 27, 128, 2, 512>>(a, threads, ld) ||
-                  lines_match<LinesFixed<18, 18, 64, 2, 512>>(a, threads, ld);
+                  lines_match<LinesFixed<18, 18, 64, 2, 512>>(a, threads, ld) ||
+                  lines_match<LinesFixed<18, 18, 256, 2, 512>>(a, threads, ld);
         return 1;
     }
     if (kind == 2) return scatter_tile_choice(g, numActive, vec, out);
