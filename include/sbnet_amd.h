@@ -193,10 +193,13 @@ int sbnet_sparse_gather_functor(const float* x, int N, int H, int W, int C, floa
    dy is the block stack of the forward op's output layout ([num_active, R, S, C], or [num_active, C, R, S] with
    transpose=1), dx a caller-allocated tensor of x's shape whose contents on entry do not matter.  With `workspace`
    (sbnet_sparse_scatter_workspace_bytes() bytes for the same geometry) and at most 2x2 blocks over a pixel, zeros
-   are written only to the pixels that no block covers, and the blocks are added in ceil(R/U)*ceil(S/V) passes
-   of mutually non-overlapping blocks, each pixel's first value stored, later ones added: reproducible, equal to the
-   composition up to fp32 reassociation of at most four addends.  Otherwise dx is cleared and the atomic
-   scatter-add runs on it.  Checks and status codes as sbnet_sparse_scatter_var. */
+   are written only to the pixels that no block covers, and one pass over the stack writes every other pixel once:
+   the block listed last over a pixel fetches the other blocks' values of it and stores 0 + their sum in list order
+   + its own.  No atomics: the result is the sequential CPU functor's (sparse_gather.cc:105-129), bit for bit, also
+   for real-valued data and signed zeros, and the same on every call.  A list that names a block twice falls back
+   to hardware atomics onto zeros; deeper overlaps take ceil(R/U)*ceil(S/V) passes of mutually non-overlapping
+   blocks (reproducible, equal to the composition up to fp32 reassociation); without workspace dx is cleared and
+   the atomic scatter-add runs on it.  Checks and status codes as sbnet_sparse_scatter_var. */
 int sbnet_sparse_gather_grad(const float* dy, int32_t num_active, const int16_t* active_block_indices, float* dx,
                              const int64_t* x_dims, int x_rank,
                              const int32_t* bsize, int bsize_len,

@@ -568,6 +568,9 @@ int sbnet_sparse_gather_grad(const float* dy, int32_t num_active, const int16_t*
     const sbnet::Geom g = make_geom((int)x_dims[0], (int)x_dims[1], (int)x_dims[2], (int)x_dims[3], bsize, bstride, boffset);
     hipStream_t s = static_cast<hipStream_t>(stream);
     bool done = false;
+    SBNET_HIP(sbnet::launch_scatter_onto_zeros(dy, dx, active_block_indices, num_active, g, transpose != 0, workspace,
+                                               workspace_bytes, s, done));
+    if (done) return SBNET_OK;
     SBNET_HIP(sbnet::launch_scatter_colored(dy, dx, active_block_indices, num_active, g, transpose != 0, workspace,
                                             workspace_bytes, s, done, true));
     if (done) return SBNET_OK;

@@ -84,6 +84,24 @@ __device__ __forceinline__ void vset(float& v, int, float f) { v = f; }
 
 template <typename T> __device__ __forceinline__ T vadd(const T& a, const T& b) { return a + b; }
 
+// 0 + a + b + c + own, with a, b and c taken in ascending order of their list positions pa, pb, pc: what a sequential
+// pass over the list leaves in a tensor of zeros.  A term that is absent comes as +0 at any position (a sum that
+// started from +0 is never -0, so adding +0 changes nothing).
+template <typename T>
+__device__ __forceinline__ T sum_in_list_order(int32_t pa, T a, int32_t pb, T b, int32_t pc, T c, const T& own, const T& zero)
+{
+    auto cx = [](int32_t& p, T& x, int32_t& q, T& y) {
+        const bool sw = p > q;
+        const int32_t p0 = sw ? q : p, q0 = sw ? p : q;
+        const T x0 = sw ? y : x, y0 = sw ? x : y;
+        p = p0; q = q0; x = x0; y = y0;
+    };
+    cx(pa, a, pb, b);
+    cx(pb, b, pc, c);
+    cx(pa, a, pb, b);
+    return vadd(vadd(vadd(vadd(zero, a), b), c), own);
+}
+
 // Streaming accesses: every byte of x, of the block stack and of the base tensor is touched once per
 // op, so loads and stores carry the nontemporal hint (measured: a plain dwordx4 copy gains ~10 %).
 template <typename T> __device__ __forceinline__ T ld_stream(const T* p) { return __builtin_nontemporal_load(p); }
@@ -207,6 +225,15 @@ constexpr int SCATTER_RANKED = 5;  // kernel-side mode; callers ask for SCATTER_
 constexpr int SCATTER_RANKED_INLINE = 6;  // kernel-side mode; callers ask for SCATTER_ASSIGN
 constexpr int RANK_ROWS_PER_THREAD = 2;   // rows of the list fetched per thread ahead of the tile's LDS phase
 
+// "Zeros plus the sum of the blocks" (the gradient of sparse_gather) in one pass over the stack, for at most 2x2
+// blocks over a pixel: k_fill_uncovered has written zeros where no block lies; every covered pixel is written once,
+// by the block listed last among those that cover it (the owner, as in SCATTER_RANKED), which fetches the other
+// blocks' values of that pixel from the stack and adds them up in list order, its own last: 0 + a + b + own, the
+// sequential CPU functor's sum (sparse_gather.cc:105-129), bit for bit, without atomics.  The neighbours' list
+// positions come from the inverse block map.  A list that names a block twice has no such map: every block then
+// adds all of its pixels with hardware atomics onto zeros (k_fill_uncovered clears everything in that case).
+constexpr int SCATTER_SUM = 7;  // kernel-side mode of sbnet_sparse_gather_grad
+
 struct ColorArgs {
     int kh, kw, pass;
     const int32_t* dup;
@@ -214,7 +241,8 @@ struct ColorArgs {
     const int32_t* rank;   // SCATTER_RANKED: nine bits per block, see k_rank_table
     // SCATTER_COLOR with `first`: the passes add onto a tensor of which only the pixels that no block covers hold
     // zeros yet (k_fill_uncovered), so a pass reads a pixel only where a block of an earlier pass has written it
-    // and stores 0 + v elsewhere.  `map` is the inverse block map [N, nBH, nBW] (list position or -1).
+    // and stores 0 + v elsewhere.  `map` is the inverse block map [N, nBH, nBW] (list position or -1); SCATTER_SUM
+    // reads it too.
     int first;
     const int32_t* map;
     int bhMin, bwMin, nBH, nBW;
@@ -280,7 +308,8 @@ __device__ __forceinline__ uint32_t rank_bits(const ColorArgs& col, uint32_t ib)
 __device__ __forceinline__ uint32_t earlier_pass_bits(const ColorArgs& col, const BlockOrigin& o)
 {
     typedef const int32_t __attribute__((address_space(4))) * const_i32_ptr;
-    // the eight neighbours' entries first (a neighbour beyond the map reads the block's own entry and is masked),
+    // the eight neighbours' entries first (a neighbour beyond the map reads the map's first entry and is masked:
+    // the block's own cell may lie beyond the map as well, when the block cannot touch the image),
     // then the arithmetic: eight independent scalar loads instead of a chain
     int32_t other[9];
     bool in[9];
@@ -289,7 +318,7 @@ __device__ __forceinline__ uint32_t earlier_pass_bits(const ColorArgs& col, cons
         const int dh = q / 3 - 1, dw = q % 3 - 1;
         const int ih = o.bh + dh - col.bhMin, iw = o.bw + dw - col.bwMin;
         in[q] = q != 4 && (unsigned)ih < (unsigned)col.nBH && (unsigned)iw < (unsigned)col.nBW;
-        const int64_t slot = ((int64_t)o.n * col.nBH + (in[q] ? ih : o.bh - col.bhMin)) * col.nBW + (in[q] ? iw : o.bw - col.bwMin);
+        const int64_t slot = in[q] ? ((int64_t)o.n * col.nBH + ih) * col.nBW + iw : 0;
         other[q] = *(const_i32_ptr)(reinterpret_cast<uintptr_t>(col.map + slot));
     }
     uint32_t bits = 0u;
@@ -304,6 +333,72 @@ __device__ __forceinline__ uint32_t earlier_pass_bits(const ColorArgs& col, cons
         }
     }
     return bits;
+}
+
+// SCATTER_SUM: the active neighbours of block ib at (o.bh, o.bw), q = 3 * (dh + 1) + (dw + 1).  `later`: nine bits
+// as in SCATTER_RANKED, the classes of the block's pixels that a neighbour listed after it covers (that neighbour,
+// or one after it, owns them).  `pos[q]`: list position of a neighbour listed before it, else -1.  All of it
+// wave-uniform (scalar loads and ALU).
+constexpr int SUM_MAX_BLOCKS = 1 << 30;
+
+struct NeighbourPos {
+    uint32_t later;
+    int32_t pos[9];
+};
+
+__device__ __forceinline__ NeighbourPos neighbour_positions(const ColorArgs& col, const BlockOrigin& o, uint32_t ib)
+{
+    typedef const int32_t __attribute__((address_space(4))) * const_i32_ptr;
+    int32_t other[9];
+    bool in[9];
+#pragma unroll
+    for (int q = 0; q < 9; ++q) {  // (independent loads; a neighbour beyond the map reads the first entry and is masked)
+        const int dh = q / 3 - 1, dw = q % 3 - 1;
+        const int ih = o.bh + dh - col.bhMin, iw = o.bw + dw - col.bwMin;
+        in[q] = q != 4 && (unsigned)ih < (unsigned)col.nBH && (unsigned)iw < (unsigned)col.nBW;
+        const int64_t slot = in[q] ? ((int64_t)o.n * col.nBH + ih) * col.nBW + iw : 0;
+        other[q] = *(const_i32_ptr)(reinterpret_cast<uintptr_t>(col.map + slot));
+    }
+    NeighbourPos nb;
+    nb.later = 0u;
+#pragma unroll
+    for (int q = 0; q < 9; ++q) {
+        const int dh = q / 3 - 1, dw = q % 3 - 1;
+        const bool active = in[q] && other[q] >= 0;
+        if (active && (uint32_t)other[q] > ib) {
+            const uint32_t rows = dh < 0 ? 1u : (dh > 0 ? 4u : 7u), cols = dw < 0 ? 1u : (dw > 0 ? 4u : 7u);
+            nb.later |= ((rows & 1u) ? cols : 0u) | ((rows & 2u) ? cols << 3 : 0u) | ((rows & 4u) ? cols << 6 : 0u);
+        }
+        nb.pos[q] = active && (uint32_t)other[q] < ib ? other[q] : -1;
+    }
+    return nb;
+}
+
+// The up to three other blocks over pixel (r, s) of the block: the vertical neighbour (dh, 0), the horizontal one
+// (0, dw) and the diagonal one (dh, dw), as list positions or -1.  In those blocks the pixel lies dh * U rows up and
+// dw * V columns left.  Meant for pixels that the block owns: every other block over them is listed before it.
+struct PixelNeighbours {
+    int32_t pv, ph, pd;
+    int dh, dw;
+};
+
+__device__ __forceinline__ PixelNeighbours pixel_neighbours(const NeighbourPos& nb, int r, int s, const Geom& g)
+{
+    PixelNeighbours p;
+    p.dh = r < g.R - g.U ? -1 : (r >= g.U ? 1 : 0);
+    p.dw = s < g.S - g.V ? -1 : (s >= g.V ? 1 : 0);
+    p.pv = p.dh < 0 ? nb.pos[1] : (p.dh > 0 ? nb.pos[7] : -1);
+    p.ph = p.dw < 0 ? nb.pos[3] : (p.dw > 0 ? nb.pos[5] : -1);
+    const int32_t upper = p.dw < 0 ? nb.pos[0] : nb.pos[2], lower = p.dw < 0 ? nb.pos[6] : nb.pos[8];
+    p.pd = p.dh != 0 && p.dw != 0 ? (p.dh < 0 ? upper : lower) : -1;
+    return p;
+}
+
+// The list names some block twice (k_pull_map's flag, written by an earlier kernel).
+__device__ __forceinline__ bool list_has_repeats(const ColorArgs& col)
+{
+    typedef const int32_t __attribute__((address_space(4))) * const_i32_ptr;
+    return *(const_i32_ptr)(reinterpret_cast<uintptr_t>(col.dup)) != 0;
 }
 
 // True when this launch has nothing to do for the block; `atomics` tells how to add otherwise.

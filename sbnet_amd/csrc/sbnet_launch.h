@@ -72,6 +72,11 @@ hipError_t launch_scatter_colored(const float* x, float* y, const int16_t* idx, 
                                   bool transpose, void* workspace, size_t workspaceBytes, hipStream_t stream,
                                   bool& done, bool ontoZeros = false);
 hipError_t launch_zero(float* y, size_t count, hipStream_t stream);
+// The same result (zeros plus the sum of overlapping blocks) in one pass over the stack: every covered pixel is
+// written once, by the block listed last over it, as the sum in list order of the blocks that cover it; at most 2x2
+// blocks over a pixel, scratch of scatter_color_workspace_bytes().
+hipError_t launch_scatter_onto_zeros(const float* x, float* y, const int16_t* idx, int numActive, const Geom& g,
+                                     bool transpose, void* workspace, size_t workspaceBytes, hipStream_t stream, bool& done);
 
 // Plain writes ("=") of overlapping blocks in the order of the sequential CPU functor: on a pixel that several
 // blocks cover, the block listed last wins (sparse_gather.cc:105-129), for either stack layout and for lists that

@@ -104,6 +104,10 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
     vec v[NHWC_UNR];
     uint32_t dst[NHWC_UNR];
     int32_t own[NHWC_UNR];
+    NeighbourPos nb;
+    nb.later = 0u;
+    const bool repeats = MODE == SCATTER_SUM && list_has_repeats(col);
+    if (MODE == SCATTER_SUM && !repeats) nb = neighbour_positions(col, o, ib);
     const rsrc_t wr = make_rsrc(MODE == SCATTER_OWNED ? col.owner + (int64_t)o.n * a.g.H * a.g.W : nullptr,
                                 MODE == SCATTER_OWNED ? (uint32_t)(a.g.H * a.g.W) * 4u : 0u);
 #pragma unroll
@@ -114,6 +118,7 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
         const int hh = o.h0 + (int)r;
         bool ok = e < a.blockV && (unsigned)hh < (unsigned)a.g.H && j >= lo && j < hi;
         if (MODE == SCATTER_RANKED) ok = ok && !ranked_out(rank_bits(col, ib), r, fdiv((uint32_t)j, a.dCV), a.g);
+        if (MODE == SCATTER_SUM) ok = ok && !ranked_out(nb.later, r, fdiv((uint32_t)j, a.dCV), a.g);
         dst[u] = ok ? (((uint32_t)hh * (uint32_t)a.g.W + (uint32_t)o.w0) * (uint32_t)CV + (uint32_t)j) * (uint32_t)(VEC * 4)
                     : BUF_OOB;
         v[u] = buf_load<VEC>(xr, ok ? e * (uint32_t)(VEC * 4) : BUF_OOB);  // off-image parts are not read
@@ -146,6 +151,42 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
         }
 #pragma unroll
         for (int u = 0; u < NHWC_UNR; ++u) buf_store<BUF_NT>(yr, dst[u], vadd(cur[u], v[u]));
+    } else if (MODE == SCATTER_SUM) {
+        if (repeats) {  // (onto zeros everywhere)
+#pragma unroll
+            for (int u = 0; u < NHWC_UNR; ++u) {
+                if (dst[u] != BUF_OOB) {
+                    float* d = img + (dst[u] >> 2);
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) atomic_add_f32(d + k, vget(v[u], k));
+                }
+            }
+            return;
+        }
+        // the owner's sum: 0 + the blocks listed before this one, in list order, + its own value; the other blocks'
+        // values of a pixel (three at most) are fetched together
+        const rsrc_t sr2 = make_rsrc(x, fdiv(a.units, a.dCpb) * a.blockV * (uint32_t)(VEC * 4));  // the whole stack
+        vec nv[NHWC_UNR][3];
+        PixelNeighbours pn[NHWC_UNR];
+#pragma unroll
+        for (int u = 0; u < NHWC_UNR; ++u) {
+            const uint32_t e = e0 + u * 64;
+            const uint32_t r = fdiv(e, a.dRow);
+            const uint32_t j = e - r * a.rowV, sc = fdiv(j, a.dCV);
+            pn[u] = pixel_neighbours(nb, (int)r, (int)sc, a.g);
+            if (dst[u] == BUF_OOB) pn[u].pv = pn[u].ph = pn[u].pd = -1;
+            const int up = pn[u].dh * a.g.U * (int)a.rowV, left = pn[u].dw * a.g.V * CV;
+            const uint32_t ev = (uint32_t)((int)e - up), eh = (uint32_t)((int)e - left), ed = (uint32_t)((int)e - up - left);
+            // (under branches: a wave without such pixels skips the load)
+            nv[u][0] = nv[u][1] = nv[u][2] = vzero<VEC>();
+            if (pn[u].pv >= 0) nv[u][0] = buf_load<VEC>(sr2, ((uint32_t)pn[u].pv * a.blockV + ev) * (uint32_t)(VEC * 4));
+            if (pn[u].ph >= 0) nv[u][1] = buf_load<VEC>(sr2, ((uint32_t)pn[u].ph * a.blockV + eh) * (uint32_t)(VEC * 4));
+            if (pn[u].pd >= 0) nv[u][2] = buf_load<VEC>(sr2, ((uint32_t)pn[u].pd * a.blockV + ed) * (uint32_t)(VEC * 4));
+        }
+#pragma unroll
+        for (int u = 0; u < NHWC_UNR; ++u)
+            buf_store<BUF_NT>(yr, dst[u], sum_in_list_order(pn[u].pv, nv[u][0], pn[u].ph, nv[u][1], pn[u].pd, nv[u][2], v[u],
+                                                            vzero<VEC>()));
     } else {
 #pragma unroll
         for (int u = 0; u < NHWC_UNR; ++u) {
@@ -236,6 +277,13 @@ __device__ __forceinline__ void scatter_planar_tile(const float* __restrict__ x,
     const BlockOrigin o = origin_of(raw, a.g);
     // (colour passes onto zeros: the neighbours' map entries, fetched while the tile's loads are in flight)
     const uint32_t ebits = MODE == SCATTER_COLOR && col.first && o.valid ? earlier_pass_bits(col, o) : 0x1ffu;
+    // (the owners' sums onto zeros: the neighbours' list positions, likewise)
+    NeighbourPos nb;
+    nb.later = 0u;
+    if (MODE == SCATTER_SUM) {
+        atomics = list_has_repeats(col);
+        if (o.valid && !atomics) nb = neighbour_positions(col, o, t.ib);
+    }
     if (MODE == SCATTER_RANKED_INLINE) {
         // nine bits: classes of this block's pixels that a block listed later covers (the later one wins them)
         uint32_t bits = 0u;
@@ -272,9 +320,12 @@ __device__ __forceinline__ void scatter_planar_tile(const float* __restrict__ x,
     // colour passes onto zeros: a pixel is read only where a block of an earlier pass has written it (an out-of-range
     // read returns 0, and 0 + v is what a pixel's first write stores)
     bool rmw[TILE_LD];
+    uint32_t rs[TILE_LD];  // SCATTER_SUM: the pixel's row and column in the block
     auto walk = [&]() {
         nhwc_walk<VEC, G>(a, t, o, tid, nthr, [&](int u, uint32_t pl, uint32_t off, uint32_t pix, uint32_t r, uint32_t sc) {
             if ((MODE == SCATTER_RANKED || MODE == SCATTER_RANKED_INLINE) && ranked_out(rbits, r, sc, a.g)) off = BUF_OOB;
+            if (MODE == SCATTER_SUM && ranked_out(nb.later, r, sc, a.g)) off = BUF_OOB;
+            rs[u] = (r << 16) | sc;
             rmw[u] = MODE != SCATTER_COLOR || ranked_out(ebits, r, sc, a.g);
             offs[u] = off;
             pls[u] = pl;
@@ -282,10 +333,45 @@ __device__ __forceinline__ void scatter_planar_tile(const float* __restrict__ x,
         });
     };
     // An add's reads of the base do not depend on the tile: they go out before the barrier, behind the tile's loads.
-    constexpr bool EARLY = MODE == SCATTER_ADD || MODE == SCATTER_COLOR;
+    // So do the reads of the other blocks' values of the pixels that this block sums (three per pixel at most).
+    constexpr bool EARLY = MODE == SCATTER_ADD || MODE == SCATTER_COLOR || MODE == SCATTER_SUM;
+    vec nv[MODE == SCATTER_SUM ? TILE_LD : 1][3];
+    PixelNeighbours pn[MODE == SCATTER_SUM ? TILE_LD : 1];
     if (EARLY) {
         walk();
-        if (!atomics) {
+        if (MODE == SCATTER_SUM) {
+            if (!atomics) {
+                const rsrc_t sr2 = make_rsrc(x, (uint32_t)a.blocks * G::C(a) * RS * 4u);  // the whole stack
+                const int S = (int)G::S(a);
+#pragma unroll
+                for (int u = 0; u < TILE_LD; ++u) {
+                    const int r = (int)(rs[u] >> 16), sc = (int)(rs[u] & 0xffffu);
+                    const int v = MODE == SCATTER_SUM ? u : 0;
+                    pn[v] = pixel_neighbours(nb, r, sc, a.g);
+                    if (offs[u] == BUF_OOB) pn[v].pv = pn[v].ph = pn[v].pd = -1;
+                    const int p = r * S + sc, up = pn[v].dh * a.g.U * S, left = pn[v].dw * a.g.V;
+                    const uint32_t c = (uint32_t)t.c0 + c0l;
+                    // (under branches, not with out-of-range offsets: few pixels have such a block at all, and a wave
+                    // that has none skips the loads, which would otherwise keep the address units as busy as real ones)
+                    nv[v][0] = nv[v][1] = nv[v][2] = vzero<VEC>();
+                    if (pn[v].pv >= 0) {
+#pragma unroll
+                        for (int k = 0; k < VEC; ++k)
+                            vset(nv[v][0], k, buf_load<1>(sr2, ((((uint32_t)pn[v].pv * G::C(a) + c + k) * RS) + (uint32_t)(p - up)) * 4u));
+                    }
+                    if (pn[v].ph >= 0) {
+#pragma unroll
+                        for (int k = 0; k < VEC; ++k)
+                            vset(nv[v][1], k, buf_load<1>(sr2, ((((uint32_t)pn[v].ph * G::C(a) + c + k) * RS) + (uint32_t)(p - left)) * 4u));
+                    }
+                    if (pn[v].pd >= 0) {
+#pragma unroll
+                        for (int k = 0; k < VEC; ++k)
+                            vset(nv[v][2], k, buf_load<1>(sr2, ((((uint32_t)pn[v].pd * G::C(a) + c + k) * RS) + (uint32_t)(p - up - left)) * 4u));
+                    }
+                }
+            }
+        } else if (!atomics) {
 #pragma unroll
             for (int u = 0; u < TILE_LD; ++u) cur[u] = buf_load<VEC>(sr, MODE == SCATTER_COLOR && !rmw[u] ? BUF_OOB : offs[u]);
         }
@@ -317,6 +403,14 @@ __device__ __forceinline__ void scatter_planar_tile(const float* __restrict__ x,
     } else if (MODE == SCATTER_ADD || (MODE == SCATTER_COLOR && !atomics)) {
 #pragma unroll
         for (int u = 0; u < TILE_LD; ++u) buf_store<BUF_NT>(yr, offs[u], vadd(cur[u], w[u]));
+    } else if (MODE == SCATTER_SUM && !atomics) {
+        // the owner's sum: 0 + the blocks listed before this one, in list order, + its own value
+#pragma unroll
+        for (int u = 0; u < TILE_LD; ++u) {
+            const int v = MODE == SCATTER_SUM ? u : 0;
+            buf_store<BUF_NT>(yr, offs[u], sum_in_list_order(pn[v].pv, nv[v][0], pn[v].ph, nv[v][1], pn[v].pd, nv[v][2], w[u],
+                                                            vzero<VEC>()));
+        }
     } else {
 #pragma unroll
         for (int u = 0; u < TILE_LD; ++u) {
@@ -750,7 +844,7 @@ static bool launch_fixed_scatter(const float* x, float* y, const float* ysrc, co
                                  int threads, size_t lds, int numActive, const ColorArgs& aux, hipStream_t stream)
 {
     if constexpr (VEC == 4 && (MODE == SCATTER_ASSIGN || MODE == SCATTER_ADD || MODE == SCATTER_RANKED ||
-                               MODE == SCATTER_RANKED_INLINE || MODE == SCATTER_COLOR)) {
+                               MODE == SCATTER_RANKED_INLINE || MODE == SCATTER_COLOR || MODE == SCATTER_SUM)) {
         // 27x27 blocks of 128 channels with 16 KB and 24 KB tiles; 16x16 blocks of 64 channels
         if constexpr (MODE == SCATTER_ASSIGN || MODE == SCATTER_RANKED_INLINE) {
             // (the 24 KB tile is what launches of few workgroups take: moved in two halves, see above)
@@ -1771,6 +1865,80 @@ hipError_t launch_scatter_owned(const float* x, float* y, const int16_t* idx, in
     if (!build_owner_map(idx, numActive, g, workspace, workspaceBytes, stream, owner)) return hipSuccess;
     done = true;
     return scatter_from(x, y, y, idx, numActive, g, transpose, SCATTER_ASSIGN, stream, owner);
+}
+
+// y = zeros, plus the sum of the blocks (the gradient of sparse_gather), for overlapping blocks of which at most 2x2
+// cover a pixel, in one pass over the stack: zeros where no block lies (k_fill_uncovered), then SCATTER_SUM.
+// `done` is false, and nothing launched, where this does not apply; the caller then takes the colour passes.
+template <int VEC>
+static void launch_sum(const float* x, float* y, const int16_t* idx, const Geom& g, int numActive, bool transpose,
+                          const ColorArgs& col, hipStream_t stream)
+{
+    if (!transpose) {
+        NhwcArgs a;
+        make_nhwc_args(g, numActive, VEC, a);
+        hipLaunchKernelGGL((k_scatter_nhwc<VEC, SCATTER_SUM>), dim3((a.units + 3) / 4), dim3(256), 0, stream, x, y,
+                           (const float*)y, idx, a, col);
+        return;
+    }
+    TileArgs a;
+    int threads;
+    size_t lds;
+    unsigned grid;
+    scatter_tile_args(g, numActive, VEC, a, threads, lds, grid);
+    if (launch_fixed_scatter<VEC, SCATTER_SUM>(x, y, y, idx, a, threads, lds, numActive, col, stream)) return;
+    hipLaunchKernelGGL((k_scatter_planar<VEC, SCATTER_SUM, TileRt>), tile_grid(a.grid2d, a.tpb, numActive, a.total, a.g),
+                       dim3(threads), lds, stream, x, y, (const float*)y, idx, a, col);
+}
+
+hipError_t launch_scatter_onto_zeros(const float* x, float* y, const int16_t* idx, int numActive, const Geom& g,
+                                     bool transpose, void* workspace, size_t workspaceBytes, hipStream_t stream, bool& done)
+{
+    done = false;
+    if (numActive <= 0 || numActive > SUM_MAX_BLOCKS || g.countDev || !(g.U < g.R || g.V < g.S)) return hipSuccess;
+    if (g.R > 32767 || g.S > 32767) return hipSuccess;  // (the tile kernel packs a pixel's row and column into a word)
+    // (the other blocks' values are read through one buffer over the whole stack: 32-bit byte offsets)
+    if ((int64_t)numActive * g.C * g.R * g.S * 4 >= (1ll << 32) - 16) return hipSuccess;
+    const size_t need = scatter_color_workspace_bytes(g, numActive);  // (the map and the flag are its first part)
+    if (!workspace || need == 0 || workspaceBytes < need || (reinterpret_cast<uintptr_t>(workspace) & 3)) return hipSuccess;
+    PullArgs pa;
+    int64_t mapN = 0;
+    if (!make_map_args(g, pa, mapN)) return hipSuccess;
+    const int vec = pick_vec(g, y, transpose ? nullptr : x);
+    FillArgs fa;
+    unsigned fillGrid = 0;
+    if (!make_fill_args(g, vec, pa, fa, fillGrid)) return hipSuccess;  // (more than 2x2 blocks over a pixel)
+    if (transpose) {
+        TileArgs a;
+        int threads;
+        size_t lds;
+        unsigned grid;
+        if ((int64_t)g.R * g.S < 4 || !scatter_tile_args(g, numActive, vec, a, threads, lds, grid)) return hipSuccess;
+    } else {
+        NhwcArgs na;
+        if (!nhwc_fits_buffers(g) || !make_nhwc_args(g, numActive, vec, na)) return hipSuccess;
+    }
+    int32_t* map = static_cast<int32_t*>(workspace);
+    int32_t* dup = map + mapN;
+    int64_t fillWgs = (mapN + 255) / 256;
+    if (fillWgs > 4096) fillWgs = 4096;
+    hipLaunchKernelGGL(k_pull_fill, dim3((unsigned)fillWgs), dim3(256), 0, stream, map, mapN, dup);
+    hipLaunchKernelGGL(k_pull_map, dim3((unsigned)((numActive + 255) / 256)), dim3(256), 0, stream, idx, numActive, pa, map, dup);
+    const int32_t* cmap = map;
+    const int32_t* cdup = dup;
+    if (vec == 4) hipLaunchKernelGGL(k_fill_uncovered<4>, dim3(fillGrid), dim3(256), 0, stream, y, cmap, cdup, fa);
+    else if (vec == 2) hipLaunchKernelGGL(k_fill_uncovered<2>, dim3(fillGrid), dim3(256), 0, stream, y, cmap, cdup, fa);
+    else hipLaunchKernelGGL(k_fill_uncovered<1>, dim3(fillGrid), dim3(256), 0, stream, y, cmap, cdup, fa);
+    ColorArgs col;
+    col.kh = 2; col.kw = 2; col.pass = 0;  // (unused by this mode, like the fields of the other orders)
+    col.dup = cdup; col.owner = nullptr; col.rank = nullptr; col.first = 0; col.map = cmap;
+    col.bhMin = pa.bhMin; col.bwMin = pa.bwMin; col.nBH = pa.nBH; col.nBW = pa.nBW;
+    col.perm = nullptr; col.counts = nullptr; col.permStride = 0;
+    if (vec == 4) launch_sum<4>(x, y, idx, g, numActive, transpose, col, stream);
+    else if (vec == 2) launch_sum<2>(x, y, idx, g, numActive, transpose, col, stream);
+    else launch_sum<1>(x, y, idx, g, numActive, transpose, col, stream);
+    done = true;
+    return hipGetLastError();
 }
 
 template <int VEC>

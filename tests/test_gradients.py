@@ -218,6 +218,33 @@ def test_gather_grad_entry_point(case):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("case", [
+    ((2, 64, 72, 32), (10, 10), (8, 8), (-1, -1)),
+    ((1, 120, 130, 128), (27, 27), (25, 25), (-1, -1)),
+    ((2, 50, 61, 24), (7, 9), (5, 6), (2, -4)),
+    ((3, 33, 47, 5), (5, 7), (3, 4), (-2, -3)),
+    ((1, 40, 40, 8), (8, 8), (4, 4), (0, 0)),                # every pixel under 2x2 blocks
+], ids=lambda c: "x".join(map(str, c[0])) + "_b%dx%d_s%dx%d" % (c[1] + c[2]))
+def test_gather_grad_sums_in_list_order(case):
+    """With at most 2x2 blocks over a pixel and no block named twice the gradient is summed without atomics, each
+    pixel as 0 + its blocks' values in list order: real-valued data (whose sums depend on the order) and signed
+    zeros come out as the sequential CPU functor leaves them, bit for bit, on every call."""
+    from sbnet_amd import ops
+    shape, bs, bst, bo = case
+    rng, idx, cnt = setup_case(case, 29, frac=0.8)
+    rng.shuffle(idx, axis=0)
+    M, C = len(idx), shape[3]
+    for transpose in (False, True):
+        gshape = (M, C, bs[0], bs[1]) if transpose else (M, bs[0], bs[1], C)
+        g = (rng.standard_normal(gshape) * 10.0 ** rng.integers(-3, 4, size=gshape)).astype(np.float32)
+        g[rng.random(gshape) < 0.05] = -0.0
+        exp = orc.sparse_gather_grad(g, shape, cnt, idx, bs, bst, bo, transpose=transpose)
+        for rep in range(2):
+            dx = ops.gather_backward(dev(g), cnt, dev(idx), shape, bs, bst, bo, transpose).cpu().numpy()
+            np.testing.assert_array_equal(dx.view(np.uint32), exp.view(np.uint32), err_msg="transpose %s" % transpose)
+
+
+@pytest.mark.gpu
 def test_chain_gather_multiply_scatter_backward():
     """x -> gather -> * w -> scatter(add) onto ybase -> sum(. * v): gradients through both Functions at once,
     against the chain rule spelled out with the oracle's pieces."""
