@@ -102,6 +102,18 @@ __device__ __forceinline__ T sum_in_list_order(int32_t pa, T a, int32_t pb, T b,
     return vadd(vadd(vadd(vadd(zero, a), b), c), own);
 }
 
+// The same where absent terms come with position -1 and value +0.  With at most one term present no order is
+// needed, and a + b + c holds two +0 terms, so it is never -0 and equals 0 + that term: the common case (pixels
+// under two blocks; only a block's corners lie under more) takes three additions and skips the sort, a wave at a time.
+template <typename T>
+__device__ __forceinline__ T sum_of_pixel(int32_t pa, const T& a, int32_t pb, const T& b, int32_t pc, const T& c, const T& own,
+                                          const T& zero)
+{
+    const int present = (int)(pa >= 0) + (int)(pb >= 0) + (int)(pc >= 0);
+    if (present >= 2) return sum_in_list_order(pa, a, pb, b, pc, c, own, zero);
+    return vadd(vadd(vadd(a, b), c), own);
+}
+
 // Streaming accesses: every byte of x, of the block stack and of the base tensor is touched once per
 // op, so loads and stores carry the nontemporal hint (measured: a plain dwordx4 copy gains ~10 %).
 template <typename T> __device__ __forceinline__ T ld_stream(const T* p) { return __builtin_nontemporal_load(p); }

@@ -185,8 +185,8 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
         }
 #pragma unroll
         for (int u = 0; u < NHWC_UNR; ++u)
-            buf_store<BUF_NT>(yr, dst[u], sum_in_list_order(pn[u].pv, nv[u][0], pn[u].ph, nv[u][1], pn[u].pd, nv[u][2], v[u],
-                                                            vzero<VEC>()));
+            buf_store<BUF_NT>(yr, dst[u], sum_of_pixel(pn[u].pv, nv[u][0], pn[u].ph, nv[u][1], pn[u].pd, nv[u][2], v[u],
+                                                       vzero<VEC>()));
     } else {
 #pragma unroll
         for (int u = 0; u < NHWC_UNR; ++u) {
@@ -227,7 +227,65 @@ __device__ __forceinline__ void scatter_planar_tile(const float* __restrict__ x,
     ListRow rows[RANK_ROWS_PER_THREAD];
     uint32_t listCount = 0;
     ListRows lr;
+    // SCATTER_SUM: the other blocks' values of the pixels that this block sums (three per pixel at most) are fetched
+    // behind the tile's own loads as well: the neighbours' list positions (scalar loads), the walk over the tile's
+    // pixels, then the loads, all before the first wait for the tile's data.
+    constexpr int NSUM = MODE == SCATTER_SUM ? TILE_LD : 1;
+    typename Vec<VEC>::type nv[NSUM][3];
+    PixelNeighbours pn[NSUM];
+    uint32_t offs[TILE_LD], pls[TILE_LD];
+    NeighbourPos nb;
+    nb.later = 0u;
+    bool summed = false;  // offs / pls / pn / nv are set
+    const uint32_t c0l = (tid & ((1u << G::lppLog(a)) - 1u)) * VEC;
+    auto fetch_neighbours = [&]() {
+        if (MODE != SCATTER_SUM) return;
+        const BlockOrigin o = origin_of(raw, a.g);
+        atomics = list_has_repeats(col);
+        if (!o.valid || atomics) return;
+        nb = neighbour_positions(col, o, t.ib);
+        summed = true;
+        const rsrc_t sr2 = make_rsrc(x, (uint32_t)a.blocks * G::C(a) * RS * 4u);  // the whole stack
+        const int S = (int)G::S(a);
+        const uint32_t c = (uint32_t)t.c0 + c0l;
+        // (wave-uniform: whole directions without a block listed earlier cost a scalar branch)
+        const bool anyV = (nb.pos[1] & nb.pos[7]) >= 0, anyH = (nb.pos[3] & nb.pos[5]) >= 0;
+        const bool anyD = (nb.pos[0] & nb.pos[2] & nb.pos[6] & nb.pos[8]) >= 0;
+        nhwc_walk<VEC, G>(a, t, o, tid, nthr, [&](int u, uint32_t pl, uint32_t off, uint32_t, uint32_t r, uint32_t sc) {
+            if (ranked_out(nb.later, r, sc, a.g)) off = BUF_OOB;  // (a block listed later owns the pixel)
+            offs[u] = off;
+            pls[u] = pl;
+            const int v = MODE == SCATTER_SUM ? u : 0;
+            pn[v].pv = pn[v].ph = pn[v].pd = -1;
+            nv[v][0] = nv[v][1] = nv[v][2] = vzero<VEC>();
+            if (!(anyV || anyH || anyD)) return;
+            const PixelNeighbours q = pixel_neighbours(nb, (int)r, (int)sc, a.g);
+            const bool mine = off != BUF_OOB;
+            const int p = (int)r * S + (int)sc, up = q.dh * a.g.U * S, left = q.dw * a.g.V;
+            // (under branches, not with out-of-range offsets: few pixels have such a block at all, and a wave
+            // that has none skips the loads, which would otherwise keep the address units as busy as real ones)
+            if (anyV && mine && q.pv >= 0) {
+                pn[v].pv = q.pv;
+#pragma unroll
+                for (int k = 0; k < VEC; ++k)
+                    vset(nv[v][0], k, buf_load<1>(sr2, ((((uint32_t)q.pv * G::C(a) + c + k) * RS) + (uint32_t)(p - up)) * 4u));
+            }
+            if (anyH && mine && q.ph >= 0) {
+                pn[v].ph = q.ph;
+#pragma unroll
+                for (int k = 0; k < VEC; ++k)
+                    vset(nv[v][1], k, buf_load<1>(sr2, ((((uint32_t)q.ph * G::C(a) + c + k) * RS) + (uint32_t)(p - left)) * 4u));
+            }
+            if (anyD && mine && q.pd >= 0) {
+                pn[v].pd = q.pd;
+#pragma unroll
+                for (int k = 0; k < VEC; ++k)
+                    vset(nv[v][2], k, buf_load<1>(sr2, ((((uint32_t)q.pd * G::C(a) + c + k) * RS) + (uint32_t)(p - up - left)) * 4u));
+            }
+        });
+    };
     auto fetch_rows = [&]() {
+        fetch_neighbours();
         if (MODE != SCATTER_RANKED_INLINE) return;
         listCount = list_count(a.g, a.blocks);
         lr = list_rows(idx, listCount);
@@ -277,13 +335,6 @@ __device__ __forceinline__ void scatter_planar_tile(const float* __restrict__ x,
     const BlockOrigin o = origin_of(raw, a.g);
     // (colour passes onto zeros: the neighbours' map entries, fetched while the tile's loads are in flight)
     const uint32_t ebits = MODE == SCATTER_COLOR && col.first && o.valid ? earlier_pass_bits(col, o) : 0x1ffu;
-    // (the owners' sums onto zeros: the neighbours' list positions, likewise)
-    NeighbourPos nb;
-    nb.later = 0u;
-    if (MODE == SCATTER_SUM) {
-        atomics = list_has_repeats(col);
-        if (o.valid && !atomics) nb = neighbour_positions(col, o, t.ib);
-    }
     if (MODE == SCATTER_RANKED_INLINE) {
         // nine bits: classes of this block's pixels that a block listed later covers (the later one wins them)
         uint32_t bits = 0u;
@@ -310,9 +361,7 @@ __device__ __forceinline__ void scatter_planar_tile(const float* __restrict__ x,
     float* img = y + (int64_t)o.n * a.imgFloats;
     const rsrc_t yr = make_rsrc(img, a.imgBytes);
     const rsrc_t sr = make_rsrc(ysrc + (int64_t)o.n * a.imgFloats, a.imgBytes);  // what an add reads
-    const uint32_t c0l = (tid & ((1u << G::lppLog(a)) - 1u)) * VEC;
     vec w[TILE_LD], cur[TILE_LD];
-    uint32_t offs[TILE_LD], pls[TILE_LD];
     int32_t own[TILE_LD];
     const rsrc_t wr = make_rsrc(MODE == SCATTER_OWNED ? col.owner + (int64_t)o.n * a.g.H * a.g.W : nullptr,
                                 MODE == SCATTER_OWNED ? (uint32_t)(a.g.H * a.g.W) * 4u : 0u);
@@ -320,12 +369,9 @@ __device__ __forceinline__ void scatter_planar_tile(const float* __restrict__ x,
     // colour passes onto zeros: a pixel is read only where a block of an earlier pass has written it (an out-of-range
     // read returns 0, and 0 + v is what a pixel's first write stores)
     bool rmw[TILE_LD];
-    uint32_t rs[TILE_LD];  // SCATTER_SUM: the pixel's row and column in the block
     auto walk = [&]() {
         nhwc_walk<VEC, G>(a, t, o, tid, nthr, [&](int u, uint32_t pl, uint32_t off, uint32_t pix, uint32_t r, uint32_t sc) {
             if ((MODE == SCATTER_RANKED || MODE == SCATTER_RANKED_INLINE) && ranked_out(rbits, r, sc, a.g)) off = BUF_OOB;
-            if (MODE == SCATTER_SUM && ranked_out(nb.later, r, sc, a.g)) off = BUF_OOB;
-            rs[u] = (r << 16) | sc;
             rmw[u] = MODE != SCATTER_COLOR || ranked_out(ebits, r, sc, a.g);
             offs[u] = off;
             pls[u] = pl;
@@ -333,45 +379,10 @@ __device__ __forceinline__ void scatter_planar_tile(const float* __restrict__ x,
         });
     };
     // An add's reads of the base do not depend on the tile: they go out before the barrier, behind the tile's loads.
-    // So do the reads of the other blocks' values of the pixels that this block sums (three per pixel at most).
-    constexpr bool EARLY = MODE == SCATTER_ADD || MODE == SCATTER_COLOR || MODE == SCATTER_SUM;
-    vec nv[MODE == SCATTER_SUM ? TILE_LD : 1][3];
-    PixelNeighbours pn[MODE == SCATTER_SUM ? TILE_LD : 1];
+    constexpr bool EARLY = MODE == SCATTER_ADD || MODE == SCATTER_COLOR;
     if (EARLY) {
         walk();
-        if (MODE == SCATTER_SUM) {
-            if (!atomics) {
-                const rsrc_t sr2 = make_rsrc(x, (uint32_t)a.blocks * G::C(a) * RS * 4u);  // the whole stack
-                const int S = (int)G::S(a);
-#pragma unroll
-                for (int u = 0; u < TILE_LD; ++u) {
-                    const int r = (int)(rs[u] >> 16), sc = (int)(rs[u] & 0xffffu);
-                    const int v = MODE == SCATTER_SUM ? u : 0;
-                    pn[v] = pixel_neighbours(nb, r, sc, a.g);
-                    if (offs[u] == BUF_OOB) pn[v].pv = pn[v].ph = pn[v].pd = -1;
-                    const int p = r * S + sc, up = pn[v].dh * a.g.U * S, left = pn[v].dw * a.g.V;
-                    const uint32_t c = (uint32_t)t.c0 + c0l;
-                    // (under branches, not with out-of-range offsets: few pixels have such a block at all, and a wave
-                    // that has none skips the loads, which would otherwise keep the address units as busy as real ones)
-                    nv[v][0] = nv[v][1] = nv[v][2] = vzero<VEC>();
-                    if (pn[v].pv >= 0) {
-#pragma unroll
-                        for (int k = 0; k < VEC; ++k)
-                            vset(nv[v][0], k, buf_load<1>(sr2, ((((uint32_t)pn[v].pv * G::C(a) + c + k) * RS) + (uint32_t)(p - up)) * 4u));
-                    }
-                    if (pn[v].ph >= 0) {
-#pragma unroll
-                        for (int k = 0; k < VEC; ++k)
-                            vset(nv[v][1], k, buf_load<1>(sr2, ((((uint32_t)pn[v].ph * G::C(a) + c + k) * RS) + (uint32_t)(p - left)) * 4u));
-                    }
-                    if (pn[v].pd >= 0) {
-#pragma unroll
-                        for (int k = 0; k < VEC; ++k)
-                            vset(nv[v][2], k, buf_load<1>(sr2, ((((uint32_t)pn[v].pd * G::C(a) + c + k) * RS) + (uint32_t)(p - up - left)) * 4u));
-                    }
-                }
-            }
-        } else if (!atomics) {
+        if (!atomics) {
 #pragma unroll
             for (int u = 0; u < TILE_LD; ++u) cur[u] = buf_load<VEC>(sr, MODE == SCATTER_COLOR && !rmw[u] ? BUF_OOB : offs[u]);
         }
@@ -381,7 +392,7 @@ __device__ __forceinline__ void scatter_planar_tile(const float* __restrict__ x,
         if (MODE == SCATTER_RANKED_INLINE) {
             for (uint32_t wv = 0; wv < (nthr >> 6); ++wv) rbits |= waveBits[wv];
         }
-        walk();
+        if (!summed) walk();
     }
 #pragma unroll
     for (int u = 0; u < TILE_LD; ++u) {
@@ -408,8 +419,8 @@ __device__ __forceinline__ void scatter_planar_tile(const float* __restrict__ x,
 #pragma unroll
         for (int u = 0; u < TILE_LD; ++u) {
             const int v = MODE == SCATTER_SUM ? u : 0;
-            buf_store<BUF_NT>(yr, offs[u], sum_in_list_order(pn[v].pv, nv[v][0], pn[v].ph, nv[v][1], pn[v].pd, nv[v][2], w[u],
-                                                            vzero<VEC>()));
+            buf_store<BUF_NT>(yr, offs[u], sum_of_pixel(pn[v].pv, nv[v][0], pn[v].ph, nv[v][1], pn[v].pd, nv[v][2], w[u],
+                                                       vzero<VEC>()));
         }
     } else {
 #pragma unroll
@@ -1896,7 +1907,6 @@ hipError_t launch_scatter_onto_zeros(const float* x, float* y, const int16_t* id
 {
     done = false;
     if (numActive <= 0 || numActive > SUM_MAX_BLOCKS || g.countDev || !(g.U < g.R || g.V < g.S)) return hipSuccess;
-    if (g.R > 32767 || g.S > 32767) return hipSuccess;  // (the tile kernel packs a pixel's row and column into a word)
     // (the other blocks' values are read through one buffer over the whole stack: 32-bit byte offsets)
     if ((int64_t)numActive * g.C * g.R * g.S * 4 >= (1ll << 32) - 16) return hipSuccess;
     const size_t need = scatter_color_workspace_bytes(g, numActive);  // (the map and the flag are its first part)
