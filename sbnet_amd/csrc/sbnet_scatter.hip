@@ -641,6 +641,41 @@ __global__ __launch_bounds__(256) void k_pull_map(const int16_t* __restrict__ id
     if (atomicCAS(map + slot, -1, ib) != -1) *dup = 1;
 }
 
+// Both steps by one workgroup, for maps and lists small enough that one workgroup is done in the time a second
+// launch takes to start.
+constexpr int BLOCK_MAP_ONE_WG = 16384;  // entries of the map, and rows of the list
+
+__global__ __launch_bounds__(1024) void k_pull_map_small(const int16_t* __restrict__ idx, int numActive, PullArgs a,
+                                                         int32_t* __restrict__ map, int mapN, int32_t* __restrict__ dup)
+{
+    const int tid = (int)threadIdx.x;
+    for (int i = tid; i < mapN; i += 1024) map[i] = -1;
+    if (tid == 0) *dup = 0;
+    __syncthreads();  // (the stores above are complete, and visible to this workgroup's atomics, beyond this point)
+    int count = numActive;
+    if (a.g.countDev) count = min(count, max(*a.g.countDev, 0));
+    for (int ib = tid; ib < count; ib += 1024) {
+        const int64_t slot = pull_slot(a, idx[(size_t)ib * 3], idx[(size_t)ib * 3 + 1], idx[(size_t)ib * 3 + 2]);
+        if (slot >= 0 && atomicCAS(map + slot, -1, ib) != -1) *dup = 1;
+    }
+}
+
+// The inverse block map of the list and its flag for repeated rows, in one launch or two.
+static void launch_block_map(const int16_t* idx, int numActive, const PullArgs& a, int32_t* map, int64_t mapN,
+                             int32_t* dup, hipStream_t stream)
+{
+    if (mapN <= BLOCK_MAP_ONE_WG && numActive <= BLOCK_MAP_ONE_WG) {
+        hipLaunchKernelGGL(k_pull_map_small, dim3(1), dim3(1024), 0, stream, idx, numActive, a, map, (int)mapN, dup);
+        return;
+    }
+    int64_t fillWgs = (mapN + 255) / 256;
+    if (fillWgs > 4096) fillWgs = 4096;
+    if (fillWgs < 1) fillWgs = 1;
+    hipLaunchKernelGGL(k_pull_fill, dim3((unsigned)fillWgs), dim3(256), 0, stream, map, mapN, dup);
+    hipLaunchKernelGGL(k_pull_map, dim3((unsigned)((numActive + 255) / 256)), dim3(256), 0, stream, idx, numActive, a, map,
+                       dup);
+}
+
 // One thread per (block, class): the up to four active blocks that cover the class's pixels, sorted by position.
 __global__ __launch_bounds__(256) void k_pull_table(const int16_t* __restrict__ idx, int numActive, PullArgs a,
                                                     const int32_t* __restrict__ map, int32_t* __restrict__ table)
@@ -1043,12 +1078,7 @@ hipError_t launch_scatter_pull(const float* x, float* y, const int16_t* idx, int
     int32_t* dup = map + mapN;
     // the table is read with 16-byte loads
     int32_t* table = reinterpret_cast<int32_t*>((reinterpret_cast<uintptr_t>(dup + 4) + 15) & ~(uintptr_t)15);
-    int64_t fillWgs = (mapN + 255) / 256;
-    if (fillWgs > 4096) fillWgs = 4096;
-    if (fillWgs < 1) fillWgs = 1;
-    const unsigned perBlockWgs = (unsigned)((numActive + 255) / 256);
-    hipLaunchKernelGGL(k_pull_fill, dim3((unsigned)fillWgs), dim3(256), 0, stream, map, mapN, dup);
-    hipLaunchKernelGGL(k_pull_map, dim3(perBlockWgs), dim3(256), 0, stream, idx, numActive, a, map, dup);
+    launch_block_map(idx, numActive, a, map, mapN, dup, stream);
     hipLaunchKernelGGL(k_pull_table, dim3((unsigned)(((int64_t)numActive * PULL_CLASSES + 255) / 256)), dim3(256), 0,
                        stream, idx, numActive, a, map, table);
     const unsigned wgs = (a.units + 3) / 4;
@@ -1310,12 +1340,7 @@ hipError_t launch_scatter_colored(const float* x, float* y, const int16_t* idx, 
     unsigned fillGrid = 0;
     // (the kernels that read only what an earlier pass wrote are the buffer-addressed ones)
     const bool partial = ontoZeros && (transpose || nhwc_fits_buffers(g)) && make_fill_args(g, vec, pa, fa, fillGrid);
-    int64_t fillWgs = (mapN + 255) / 256;
-    if (fillWgs > 4096) fillWgs = 4096;
-    if (fillWgs < 1) fillWgs = 1;
-    hipLaunchKernelGGL(k_pull_fill, dim3((unsigned)fillWgs), dim3(256), 0, stream, map, mapN, dup);
-    hipLaunchKernelGGL(k_pull_map, dim3((unsigned)((numActive + 255) / 256)), dim3(256), 0, stream, idx, numActive, pa,
-                       map, dup);
+    launch_block_map(idx, numActive, pa, map, mapN, dup, stream);
     if (sorted)
         hipLaunchKernelGGL(k_color_sort, dim3(1), dim3(1024), 0, stream, idx, numActive, g, col.kh, col.kw,
                            (const int32_t*)dup, counts, perm, numActive);
@@ -1930,10 +1955,7 @@ hipError_t launch_scatter_onto_zeros(const float* x, float* y, const int16_t* id
     }
     int32_t* map = static_cast<int32_t*>(workspace);
     int32_t* dup = map + mapN;
-    int64_t fillWgs = (mapN + 255) / 256;
-    if (fillWgs > 4096) fillWgs = 4096;
-    hipLaunchKernelGGL(k_pull_fill, dim3((unsigned)fillWgs), dim3(256), 0, stream, map, mapN, dup);
-    hipLaunchKernelGGL(k_pull_map, dim3((unsigned)((numActive + 255) / 256)), dim3(256), 0, stream, idx, numActive, pa, map, dup);
+    launch_block_map(idx, numActive, pa, map, mapN, dup, stream);
     const int32_t* cmap = map;
     const int32_t* cdup = dup;
     if (vec == 4) hipLaunchKernelGGL(k_fill_uncovered<4>, dim3(fillGrid), dim3(256), 0, stream, y, cmap, cdup, fa);
