@@ -1435,6 +1435,29 @@ __global__ __launch_bounds__(256) void k_cell_map(const int16_t* __restrict__ id
     chain[ib] = prev;
 }
 
+// The cleared map and the list's rows in it by one workgroup, for maps and lists small enough that one workgroup
+// is done in the time a second launch takes to start.
+__global__ __launch_bounds__(1024) void k_cell_map_small(const int16_t* __restrict__ idx, int numActive, StripArgs a,
+                                                          int32_t* __restrict__ map, int mapN,
+                                                          int32_t* __restrict__ chain, int32_t* __restrict__ dup)
+{
+    const int tid = (int)threadIdx.x;
+    for (int i = tid; i < mapN; i += 1024) map[i] = -1;
+    if (tid == 0) *dup = 0;
+    __syncthreads();  // (the stores above are complete, and visible to this workgroup's atomics, beyond this point)
+    int count = numActive;
+    if (a.g.countDev) count = min(count, max(*a.g.countDev, 0));
+    for (int ib = tid; ib < count; ib += 1024) {
+        const int64_t slot = cell_slot(a, idx[(size_t)ib * 3], idx[(size_t)ib * 3 + 1], idx[(size_t)ib * 3 + 2]);
+        int32_t prev = -1;
+        if (slot >= 0) {
+            prev = atomicExch(map + slot, ib);
+            if (prev >= 0) *dup = 1;
+        }
+        chain[ib] = prev;
+    }
+}
+
 // VEC channels of block ib at block pixel (r, s), channel vector cv.
 template <int VEC, bool PLANAR>
 __device__ __forceinline__ typename Vec<VEC>::type strip_stack_load(const float* __restrict__ x, int ib, int r,
@@ -2018,11 +2041,16 @@ hipError_t launch_scatter_over_base(const float* x, const float* ybase, float* y
             int32_t* map = static_cast<int32_t*>(workspace);
             int32_t* dup = map + mapN;
             int32_t* chain = dup + 4;
-            int64_t fillWgs = (mapN + 255) / 256;
-            if (fillWgs > 4096) fillWgs = 4096;
-            hipLaunchKernelGGL(k_pull_fill, dim3((unsigned)fillWgs), dim3(256), 0, stream, map, mapN, dup);
-            hipLaunchKernelGGL(k_cell_map, dim3((unsigned)((numActive + 255) / 256)), dim3(256), 0, stream, idx, numActive,
-                               a, map, chain, dup);
+            if (mapN <= BLOCK_MAP_ONE_WG && numActive <= BLOCK_MAP_ONE_WG) {
+                hipLaunchKernelGGL(k_cell_map_small, dim3(1), dim3(1024), 0, stream, idx, numActive, a, map, (int)mapN,
+                                   chain, dup);
+            } else {
+                int64_t fillWgs = (mapN + 255) / 256;
+                if (fillWgs > 4096) fillWgs = 4096;
+                hipLaunchKernelGGL(k_pull_fill, dim3((unsigned)fillWgs), dim3(256), 0, stream, map, mapN, dup);
+                hipLaunchKernelGGL(k_cell_map, dim3((unsigned)((numActive + 255) / 256)), dim3(256), 0, stream, idx,
+                                   numActive, a, map, chain, dup);
+            }
             const int op = transpose && !planar ? STRIP_COPY : (mode == SCATTER_ADD ? STRIP_ADD : STRIP_ASSIGN);
             if (vec == 4) launch_strip<4>(x, ybase, y, planar, op, map, chain, dup, a, stream);
             else if (vec == 2) launch_strip<2>(x, ybase, y, planar, op, map, chain, dup, a, stream);
