@@ -1678,6 +1678,123 @@ __global__ __launch_bounds__(256) void k_scatter_strip(const float* __restrict__
     }
 }
 
+// ---- planar stack, blocks that tile the plane (bsize == bstride): one launch over the cells --------------------
+//
+// A planar stack whose rows the strips above cannot stage (18x18 blocks at an odd offset: 72-byte pieces at 8-byte
+// alignment) wants to be read along its planes, by the tile kernel.  With bsize == bstride a cell is exactly its
+// block, so the launch runs over the CELLS of the grid instead of the list: a workgroup looks its cell up in the
+// map; an active cell is scattered as one tile of scatter_planar_tile (which reads the base where it adds), an
+// empty cell is copied from the base, tile number `rem` of its `tpb` taking every tpb-th part of the cell's row
+// segments.  Every byte of the output is written once and nothing is read twice.  A cell that several rows of the
+// list name (rare) is built element by element: the row listed last for a plain write, every row in list order
+// for an add (sparse_gather.cc:105-129).
+struct CellArgs {
+    int bhMin, bwMin, nBH, nBW;
+    uint32_t CV;  // channel vectors per pixel
+    FastDiv dBW, dBHW;
+};
+
+constexpr int CELL_UNR = 4;
+
+template <int VEC, int MODE>
+__device__ __forceinline__ void cell_by_elements(const float* __restrict__ x, const float* __restrict__ ybase,
+                                                 float* __restrict__ y, const int32_t* __restrict__ chain,
+                                                 const TileArgs& a, const CellArgs& c, int head, uint32_t cell,
+                                                 uint32_t rem)
+{
+    typedef typename Vec<VEC>::type vec;
+    const Geom& g = a.g;
+    const uint32_t n = fdiv(cell, c.dBHW);
+    const uint32_t inImg = cell - n * (uint32_t)(c.nBH * c.nBW);
+    const uint32_t ih = fdiv(inImg, c.dBW), iw = inImg - ih * (uint32_t)c.nBW;
+    const int h0 = g.oh + ((int)ih + c.bhMin) * g.U, w0 = g.ow + ((int)iw + c.bwMin) * g.V;
+    const int hlo = max(0, h0), hhi = min(g.H, h0 + g.U), wlo = max(0, w0), whi = min(g.W, w0 + g.V);
+    if (hhi <= hlo || whi <= wlo) return;
+    const uint32_t segV = (uint32_t)(whi - wlo) * c.CV;  // vectors per row segment: contiguous in the tensor
+    const uint32_t total = (uint32_t)(hhi - hlo) * segV;
+    const uint32_t nthr = blockDim.x, stride = a.tpb * nthr;
+    const rsrc_t br = make_rsrc(ybase + (int64_t)n * a.imgFloats, a.imgBytes);
+    const rsrc_t yr = make_rsrc(y + (int64_t)n * a.imgFloats, a.imgBytes);
+    if (head < 0) {
+        for (uint32_t e0 = rem * nthr + threadIdx.x; e0 < total; e0 += CELL_UNR * stride) {
+            uint32_t off[CELL_UNR];
+            vec v[CELL_UNR];
+#pragma unroll
+            for (int u = 0; u < CELL_UNR; ++u) {
+                const uint32_t e = e0 + (uint32_t)u * stride;
+                const uint32_t r = e / segV, j = e - r * segV;
+                off[u] = e < total ? ((((uint32_t)hlo + r) * (uint32_t)g.W + (uint32_t)wlo) * c.CV + j) * (uint32_t)(VEC * 4)
+                                   : BUF_OOB;
+                v[u] = buf_load<VEC>(br, off[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < CELL_UNR; ++u) buf_store<BUF_NT>(yr, off[u], v[u]);
+        }
+        return;
+    }
+    // several rows of the list name this cell
+    const int64_t plane = (int64_t)g.R * g.S;
+    int last = head;
+    for (int q = head; q >= 0; q = chain[q]) last = max(last, q);
+    for (uint32_t e = rem * nthr + threadIdx.x; e < total; e += stride) {
+        const uint32_t r = e / segV, j = e - r * segV;
+        const uint32_t px = j / c.CV, cv = j - px * c.CV;
+        const uint32_t off = ((((uint32_t)hlo + r) * (uint32_t)g.W + (uint32_t)wlo) * c.CV + j) * (uint32_t)(VEC * 4);
+        const int64_t at = ((int64_t)hlo + r - h0) * g.S + ((int64_t)wlo + px - w0);  // the pixel inside the block's plane
+        vec out;
+        if (MODE == SCATTER_ADD) {
+            out = buf_load<VEC>(br, off);
+            int prev = -1;
+            for (;;) {
+                int cur = 0x7fffffff;
+                for (int q = head; q >= 0; q = chain[q])
+                    if (q > prev && q < cur) cur = q;
+                if (cur == 0x7fffffff) break;
+                const float* __restrict__ src = x + ((int64_t)cur * g.C + cv * VEC) * plane + at;
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) vset(out, k, vget(out, k) + src[k * plane]);
+                prev = cur;
+            }
+        } else {
+            const float* __restrict__ src = x + ((int64_t)last * g.C + cv * VEC) * plane + at;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) vset(out, k, src[k * plane]);
+        }
+        buf_store<BUF_NT>(yr, off, out);
+    }
+}
+
+template <int VEC, int MODE>
+__global__ __launch_bounds__(512) void k_scatter_cells(const float* __restrict__ x, const float* ybase, float* y,
+                                                       const int16_t* __restrict__ idx,
+                                                       const int32_t* __restrict__ map,
+                                                       const int32_t* __restrict__ chain,
+                                                       const int32_t* __restrict__ dup, TileArgs a, ColorArgs col,
+                                                       CellArgs c)
+{
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    __shared__ uint32_t waveBits[8];
+    typedef const int32_t __attribute__((address_space(4))) * const_i32_ptr;
+    uint32_t cell, rem;
+    if (a.grid2d) {
+        cell = blockIdx.y;
+        rem = blockIdx.x;
+    } else {
+        cell = blockIdx.x / a.tpb;
+        rem = blockIdx.x - cell * a.tpb;
+    }
+    // (scalar loads: the map was written by an earlier launch and is not written here)
+    const int head = ((const_i32_ptr)(reinterpret_cast<uintptr_t>(map)))[cell];
+    const bool dups = *(const_i32_ptr)(reinterpret_cast<uintptr_t>(dup)) != 0;
+    bool several = false;
+    if (dups && head >= 0) several = ((const_i32_ptr)(reinterpret_cast<uintptr_t>(chain)))[head] >= 0;
+    if (head >= 0 && !several) {
+        scatter_planar_tile<VEC, MODE, TileRt>(x, y, ybase, idx, a, col, lds, waveBits, (uint32_t)head, rem);
+        return;
+    }
+    cell_by_elements<VEC, MODE>(x, ybase, y, chain, a, c, head, cell, rem);
+}
+
 struct CoverArgs {
     Geom g;
     uint32_t RS;
@@ -2012,6 +2129,40 @@ static void launch_strip(const float* x, const float* ybase, float* y, bool plan
 #undef SBNET_STRIP
 }
 
+// The copying scatter of a planar stack as one launch over the cells (k_scatter_cells); false, with nothing
+// launched, where that does not apply: blocks that do not tile the plane, cells too small to be copied one by one.
+template <int VEC>
+static bool launch_cells(const float* x, const float* ybase, float* y, const int16_t* idx, int numActive, const Geom& g,
+                         ScatterMode mode, const StripArgs& sa, int64_t mapN, const int32_t* map, const int32_t* chain,
+                         const int32_t* dup, hipStream_t stream, bool dry)
+{
+    if (g.R != g.U || g.S != g.V || (int64_t)g.R * g.S < 4) return false;
+    if ((int64_t)g.U * g.V * g.C * 4 < 4096 || mapN > 0x7fffffffll) return false;
+    TileArgs a;
+    int threads;
+    size_t lds;
+    unsigned grid;
+    if (!scatter_tile_args(g, (int)mapN, VEC, a, threads, lds, grid)) return false;
+    if (mapN * (int64_t)a.tpb >= (1ll << 31)) return false;
+    if (dry) return true;
+    a.grid2d = mapN <= GRID_Y_MAX;
+    CellArgs c;
+    c.bhMin = sa.bhMin; c.bwMin = sa.bwMin; c.nBH = sa.nBH; c.nBW = sa.nBW;
+    c.CV = (uint32_t)(g.C / VEC);
+    c.dBW = make_fastdiv((uint32_t)sa.nBW);
+    c.dBHW = make_fastdiv((uint32_t)(sa.nBH * sa.nBW));
+    const ColorArgs aux{1, 1, 0, nullptr, nullptr, nullptr, 0, nullptr, 0, 0, 0, 0, nullptr, nullptr, 0};
+    const dim3 gr = a.grid2d ? dim3(a.tpb, (unsigned)mapN) : dim3((unsigned)(mapN * a.tpb));
+    (void)numActive;
+    if (mode == SCATTER_ADD)
+        hipLaunchKernelGGL((k_scatter_cells<VEC, SCATTER_ADD>), gr, dim3(threads), lds, stream, x, ybase, y, idx, map, chain,
+                           dup, a, aux, c);
+    else
+        hipLaunchKernelGGL((k_scatter_cells<VEC, SCATTER_ASSIGN>), gr, dim3(threads), lds, stream, x, ybase, y, idx, map,
+                           chain, dup, a, aux, c);
+    return true;
+}
+
 hipError_t launch_scatter_over_base(const float* x, const float* ybase, float* y, const int16_t* idx, int numActive,
                                     const Geom& g, bool transpose, ScatterMode mode, void* workspace,
                                     size_t workspaceBytes, hipStream_t stream, bool& done)
@@ -2030,11 +2181,17 @@ hipError_t launch_scatter_over_base(const float* x, const float* ybase, float* y
         const size_t need = scatter_cover_workspace_bytes(g, numActive);
         bool planar = transpose;
         bool ok = need != 0 && workspaceBytes >= need;
+        bool cells = false;  // one launch over the cells of the block grid instead of the strips
         if (ok && !make_strip_args(g, vec, planar, x, a, mapN)) {
             planar = false;
-            // (two passes and four launches: worth it once the blocks cover enough of the tensor)
-            ok = transpose && (int64_t)numActive * g.R * g.S * g.C * 4 >= (16ll << 20) &&
-                 make_strip_args(g, vec, false, x, a, mapN);
+            ok = transpose && make_strip_args(g, vec, false, x, a, mapN);
+            if (ok) {
+                cells = vec == 4 ? launch_cells<4>(x, ybase, y, idx, numActive, g, mode, a, mapN, nullptr, nullptr, nullptr, stream, true)
+                      : vec == 2 ? launch_cells<2>(x, ybase, y, idx, numActive, g, mode, a, mapN, nullptr, nullptr, nullptr, stream, true)
+                                 : launch_cells<1>(x, ybase, y, idx, numActive, g, mode, a, mapN, nullptr, nullptr, nullptr, stream, true);
+                // (else two passes and four launches: worth it once the blocks cover enough of the tensor)
+                if (!cells) ok = (int64_t)numActive * g.R * g.S * g.C * 4 >= (16ll << 20);
+            }
         }
         if (ok) {
             a.g = g;
@@ -2050,6 +2207,13 @@ hipError_t launch_scatter_over_base(const float* x, const float* ybase, float* y
                 hipLaunchKernelGGL(k_pull_fill, dim3((unsigned)fillWgs), dim3(256), 0, stream, map, mapN, dup);
                 hipLaunchKernelGGL(k_cell_map, dim3((unsigned)((numActive + 255) / 256)), dim3(256), 0, stream, idx,
                                    numActive, a, map, chain, dup);
+            }
+            if (cells) {
+                if (vec == 4) launch_cells<4>(x, ybase, y, idx, numActive, g, mode, a, mapN, map, chain, dup, stream, false);
+                else if (vec == 2) launch_cells<2>(x, ybase, y, idx, numActive, g, mode, a, mapN, map, chain, dup, stream, false);
+                else launch_cells<1>(x, ybase, y, idx, numActive, g, mode, a, mapN, map, chain, dup, stream, false);
+                done = true;
+                return hipGetLastError();
             }
             const int op = transpose && !planar ? STRIP_COPY : (mode == SCATTER_ADD ? STRIP_ADD : STRIP_ASSIGN);
             if (vec == 4) launch_strip<4>(x, ybase, y, planar, op, map, chain, dup, a, stream);

@@ -511,7 +511,11 @@ def test_host_visible_count_is_never_stale_and_threads_do_not_mix():
     ((1, 512, 512, 30), (9, 9), (9, 9), (-4, 3), 0.95, True),        # 8-byte vectors
     ((1, 1200, 1100, 7), (11, 13), (11, 13), (0, 0), 1.0, True),     # 4-byte vectors
     ((1, 800, 800, 32), (27, 27), (25, 25), (-1, -1), 0.9, False),   # plane split over several tiles
-], ids=lambda g: "x".join(map(str, g[0])) + "_b%dx%d" % g[1])
+    ((1, 300, 480, 64), (18, 18), (18, 18), (-1, -2), 0.5, True),    # planar stack: one launch over the cells,
+    ((1, 300, 480, 64), (18, 18), (18, 18), (-1, -2), 0.5, False),   # half of them empty
+    ((2, 150, 130, 256), (18, 18), (18, 18), (-1, -2), 0.3, False),  # several channel chunks
+    ((1, 4500, 4000, 4), (16, 17), (16, 17), (-7, -11), 0.7, True),  # more cells than a launch has rows
+], ids=lambda g: "x".join(map(str, g[0])) + "_b%dx%d_%s" % (g[1] + ("add" if g[5] else "assign",)))
 def test_copying_scatter_moves_every_byte_once(geom):
     """sparse_scatter (the op that returns a new tensor) with enough coverage builds its output from two disjoint
     parts -- pixels no active block covers are copied from ybase, covered ones written by the scatter, which
@@ -523,7 +527,8 @@ def test_copying_scatter_moves_every_byte_once(geom):
     allb = np.array([(n, i, j) for n in range(N) for i in range(bc[0]) for j in range(bc[1])], np.int16)
     idx = allb[rng.random(len(allb)) < keep]
     cnt = np.array([len(idx)], np.int32)
-    assert len(idx) * bs[0] * bs[1] * C * 4 >= 16 << 20   # enough coverage for the one-pass path
+    # enough coverage for the one-pass path (the launch over cells of blocks that tile the plane needs none)
+    assert len(idx) * bs[0] * bs[1] * C * 4 >= 16 << 20 or tuple(bs) == tuple(bst)
     x = rng.standard_normal((N, H, W, C)).astype(np.float32)
     base = rng.standard_normal((N, H, W, C)).astype(np.float32)
     idx_d, cnt_t, base_d = dev(idx), torch.from_numpy(cnt), dev(base)
@@ -553,6 +558,8 @@ def test_copying_scatter_moves_every_byte_once(geom):
     ((1, 64, 64, 64), (8, 8), (8, 8), (-3, 0)),     # two channel chunks, rows offset
     ((2, 30, 44, 16), (3, 4), (5, 8), (1, 0)),      # gaps between the blocks
     ((1, 33, 47, 5), (5, 7), (6, 7), (-2, -3)),     # scalar channel vectors, nothing aligned
+    ((1, 70, 90, 48), (9, 10), (9, 10), (-2, -3)),  # planar stack by cells: blocks that tile the plane, odd offset
+    ((2, 50, 41, 6), (13, 15), (13, 15), (0, -1)),  # the same with 8-byte channel vectors
 ])
 def test_copying_scatter_of_a_list_with_repeated_rows(geom):
     """Non-overlapping blocks, a list that names some blocks twice or three times with different stack rows: the
@@ -567,8 +574,10 @@ def test_copying_scatter_of_a_list_with_repeated_rows(geom):
     M = len(idx)
     cnt = np.array([M], np.int32)
     base = rng.standard_normal((N, H, W, C)).astype(np.float32)
+    # planar stacks are exact for such lists where the strips stage them or the launch runs over the cells
     aligned = bs[1] % 4 == 0 and bst[1] % 4 == 0 and bo[1] % bst[1] == 0
-    for transpose in ((False, True) if aligned else (False,)):
+    by_cells = tuple(bs) == tuple(bst) and bst[0] * bst[1] * C * 4 >= 4096
+    for transpose in ((False, True) if aligned or by_cells else (False,)):
         shape = (M, C, bs[0], bs[1]) if transpose else (M, bs[0], bs[1], C)
         stack = (rng.standard_normal(shape) * rng.choice([1e-3, 1.0, 1e4], size=(M, 1, 1, 1))).astype(np.float32)
         for add in (False, True):
