@@ -64,7 +64,8 @@ def parse():
     ap.add_argument("--density", type=float, default=0.30)
     ap.add_argument("--all-configs", action="store_true")
     ap.add_argument("--only", default=None, metavar="NAME",
-                    help="time one configuration only (C1, C2, C3@5%%, C3@15%%, C3@30%%, C4, C5) and print its row to "
+                    help="time one configuration only (C1, C2, C3@5%%, C3@15%%, C3@30%%, C4, C5, or `layers` for the reference's "
+                         "layer shapes) and print its row to "
                          "stdout instead of the benchmark line: for profiling the other configurations' kernels")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline (profiling runs)")
     ap.add_argument("--ops-only", action="store_true",
@@ -497,6 +498,9 @@ def main():
         del src, dst
         torch.cuda.empty_cache()
 
+    if args.only == "layers":
+        print(json.dumps(layer_rows(torch, lib, workloads)))
+        return
     if args.only:
         if args.only not in CONFIGS:
             print("bench.py: --only takes one of %s" % ", ".join(CONFIGS), file=sys.stderr)
@@ -659,22 +663,7 @@ def main():
     # the other benchmark configurations, each end to end (host-visible count) and per op
     out["configs"] = {name: config_row(name, torch, lib, workloads) for name in ("C1", "C2", "C4", "C5")}
 
-    # the shapes the reference's own test times its gather + scatter on (timed region: both ops)
-    layers = {}
-    for size in workloads.REFERENCE_LAYER_SIZES:
-        for transpose in (False, True):
-            p = Path(workloads.reference_layer(size, transpose), torch, lib, nsets=3)
-            t = p.op_table()
-            layers["%dx%dx%d %s" % (size + ("transpose" if transpose else "nhwc",))] = {
-                "M": p.M, "gather": t["gather"], "scatter": t["scatter"],
-                "gather_plus_scatter_us": round(t["gather"]["us"] + t["scatter"]["us"], 2)}
-            del p
-            torch.cuda.empty_cache()
-    out["reference_layer_sizes"] = {
-        "note": "benchmarkLayerSizes of the reference's test (18x18 blocks at stride 18, offset (-1,-2), every block "
-                "active): sparse_gather, then the copying sparse_scatter(add=False); the reference times both ops "
-                "together with its in-graph timers",
-        "rows": layers}
+    out["reference_layer_sizes"] = layer_rows(torch, lib, workloads)
     print(json.dumps(out))
     sys.stdout.flush()
 
@@ -685,6 +674,24 @@ def main():
 
 
 CONFIGS = ["C1", "C2", "C3@5%", "C3@15%", "C3@30%", "C4", "C5"]
+
+
+def layer_rows(torch, lib, workloads):
+    """The shapes the reference's own test times its gather + scatter on (timed region: both ops)."""
+    layers = {}
+    for size in workloads.REFERENCE_LAYER_SIZES:
+        for transpose in (False, True):
+            p = Path(workloads.reference_layer(size, transpose), torch, lib, nsets=3)
+            t = p.op_table()
+            layers["%dx%dx%d %s" % (size + ("transpose" if transpose else "nhwc",))] = {
+                "M": p.M, "gather": t["gather"], "scatter": t["scatter"],
+                "gather_plus_scatter_us": round(t["gather"]["us"] + t["scatter"]["us"], 2)}
+            del p
+            torch.cuda.empty_cache()
+    return {"note": "benchmarkLayerSizes of the reference's test (18x18 blocks at stride 18, offset (-1,-2), every block "
+                    "active): sparse_gather, then the copying sparse_scatter(add=False); the reference times both ops "
+                    "together with its in-graph timers",
+            "rows": layers}
 
 
 def config_row(name, torch, lib, workloads):
