@@ -322,7 +322,8 @@ class BenchSet(ctypes.Structure):   # struct sbnet_bench_set of sbnet_amd/csrc/s
     _fields_ = [("mask", ctypes.c_void_p), ("x", ctypes.c_void_p), ("base", ctypes.c_void_p),
                 ("stack", ctypes.c_void_p), ("idx", ctypes.c_void_p), ("count_dev", ctypes.c_void_p),
                 ("reduce_ws", ctypes.c_void_p), ("reduce_ws_bytes", ctypes.c_size_t),
-                ("scatter_ws", ctypes.c_void_p), ("scatter_ws_bytes", ctypes.c_size_t)]
+                ("scatter_ws", ctypes.c_void_p), ("scatter_ws_bytes", ctypes.c_size_t),
+                ("scatter_stack", ctypes.c_void_p), ("out", ctypes.c_void_p)]
 
 
 class BenchGeom(ctypes.Structure):  # struct sbnet_bench_geom
@@ -330,12 +331,14 @@ class BenchGeom(ctypes.Structure):  # struct sbnet_bench_geom
                 ("bcount", I2), ("bsize", I2), ("bstride", I2), ("boffset", I2),
                 ("s_bsize", I2), ("s_bstride", I2), ("s_boffset", I2),
                 ("tol", ctypes.c_float), ("avgpool", ctypes.c_int), ("transpose", ctypes.c_int),
-                ("add", ctypes.c_int), ("atomic", ctypes.c_int), ("max_active", ctypes.c_int32)]
+                ("add", ctypes.c_int), ("atomic", ctypes.c_int), ("max_active", ctypes.c_int32),
+                ("fixed_count", ctypes.c_int32)]
 
 
-def cxx_pipeline(path, steps, warmup, batches):
+def cxx_pipeline(path, steps, warmup, batches, device_count=True):
     """The step driven by a C++ host loop over the same C ABI (libsbnet_bench.so): ms per step of the median batch,
-    for the reference's contract (mode 0, count handed to the host) and with the count on the device (mode 1)."""
+    for the reference's contract (mode 0, count handed to the host) and, for the in-place pipeline, with the count
+    on the device (mode 1).  Workloads without a mask or without x skip those ops; the copying op writes `out`."""
     so = os.path.join(ROOT, "sbnet_amd", "libsbnet_bench.so")
     if not os.path.exists(so):
         raise RuntimeError("%s is not built; run `make -C sbnet_amd/csrc`" % so)
@@ -350,20 +353,24 @@ def cxx_pipeline(path, steps, warmup, batches):
                      ctypes.c_void_p, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int32)]
     wl, torch = path.wl, path.torch
     R, S = wl.bsize
+    ptr = lambda t: t.data_ptr() if t is not None else None
+    # the gathered stack at the list's capacity (the device-count launches cover all of it) where a gather runs
     caps = [torch.empty((path.maxidx, path.C, R, S) if wl.transpose else (path.maxidx, R, S, path.C),
-                        dtype=torch.float32, device="cuda:0") for _ in path.sets]
+                        dtype=torch.float32, device="cuda:0") if s["x"] is not None else None for s in path.sets]
     sets = (BenchSet * len(path.sets))()
     for k, s in enumerate(path.sets):
         sws = s["sws"]
-        sets[k] = BenchSet(s["mask"].data_ptr(), s["x"].data_ptr(), s["base"].data_ptr(), caps[k].data_ptr(),
+        # the scatter reads the gathered stack where both ops share a block size, else a stack of its own size
+        sstack = caps[k] if s.get("stack") is not None and s["sstack"] is s["stack"] else s["sstack"]
+        sets[k] = BenchSet(ptr(s["mask"]), ptr(s["x"]), s["base"].data_ptr(), ptr(caps[k]),
                            s["idx"].data_ptr(), s["dcount"].data_ptr(), s["ws"].data_ptr(), path.nws,
-                           sws.data_ptr() if sws is not None else None, sws.numel() if sws is not None else 0)
+                           ptr(sws), sws.numel() if sws is not None else 0, sstack.data_ptr(), ptr(s.get("out")))
     g = BenchGeom(path.N, path.H, path.W, path.C, I2(*wl.bcount), I2(*wl.bsize), I2(*wl.bstride), I2(*wl.boffset),
                   I2(*wl.s_bsize), I2(*wl.s_bstride), I2(*wl.s_boffset), wl.tol, int(wl.avgpool), int(wl.transpose),
-                  int(wl.s_add), int(wl.s_atomic), path.maxidx)
+                  int(wl.s_add), int(wl.s_atomic), path.maxidx, path.M)
     out = {}
     sec, cnt = ctypes.c_double(0.0), ctypes.c_int32(0)
-    for mode, name in ((0, "host_count"), (1, "device_count")):
+    for mode, name in ((0, "host_count"), (1, "device_count"))[:2 if device_count else 1]:
         path.check(loop(sets, len(path.sets), ctypes.byref(g), max(warmup, len(path.sets)), mode, path.stream,
                         ctypes.byref(sec), ctypes.byref(cnt)))
         per = []
@@ -712,7 +719,9 @@ def config_row(name, torch, lib, workloads):
     torch.cuda.synchronize()
     e2e = (time.perf_counter() - t0) / K * 1e6
     wl = p.wl
-    row = {"config": name, "M": p.M, "end_to_end_us": round(e2e, 1), "ops": p.op_table(),
+    cxx = cxx_pipeline(p, K, 5, 5, device_count=False)["host_count"] * 1e3
+    row = {"config": name, "M": p.M, "end_to_end_us": round(e2e, 1), "end_to_end_cxx_us": round(cxx, 1),
+           "ops": p.op_table(),
            "workload": "x=%s bsize %s bstride %s boffset %s %s-pool tol %g; gather transpose=%s; %s add=%s atomic=%s "
                        "bsize %s bstride %s boffset %s" % (
                            wl.shape, wl.bsize, wl.bstride, wl.boffset, "avg" if wl.avgpool else "max", wl.tol,

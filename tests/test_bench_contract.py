@@ -65,5 +65,5 @@ def test_bench_structs_match_the_cxx_loop():
     so = os.path.join(ROOT, "sbnet_amd", "libsbnet_bench.so")
     lib = ctypes.CDLL(so)
     lib.sbnet_bench_struct_bytes.restype = ctypes.c_size_t
-    assert lib.sbnet_bench_struct_bytes(0) == ctypes.sizeof(bench.BenchSet) == 80
+    assert lib.sbnet_bench_struct_bytes(0) == ctypes.sizeof(bench.BenchSet) == 96
     assert lib.sbnet_bench_struct_bytes(1) == ctypes.sizeof(bench.BenchGeom)
