@@ -234,14 +234,14 @@ size_t sbnet_sparse_scatter_workspace_bytes(int32_t num_active, const int64_t* y
  *   add=0 with overlapping blocks (bstride < bsize): the reference's CPU functor walks the list front to
  *   back, so the block listed last wins on a pixel that several blocks cover (sparse_gather.cc:105-129).
  *   This library writes exactly that, for both stack layouts and for lists that name a block twice: without
- *   scratch when the stack is planar (transpose=1), at most 2x2 blocks cover a pixel (bsize <= 2*bstride) and
- *   the list has at most 2048 blocks (the kernel that moves a block compares it with the rows listed after
- *   it); otherwise given scratch (below).  Where neither holds, as in the reference's GPU path, which block
- *   wins is unspecified unless the overlapping values are equal.
+ *   scratch when at most 2x2 blocks cover a pixel (bsize <= 2*bstride) and the list has at most 2048 blocks
+ *   (planar stack, transpose=1) or 192 blocks (NHWC stack): the kernel that moves a block compares it with
+ *   the rows listed after it; otherwise given scratch (below).  Where neither holds, as in the reference's
+ *   GPU path, which block wins is unspecified unless the overlapping values are equal.
  *   workspace   optional device scratch (4-byte aligned) of sbnet_sparse_scatter_workspace_bytes() bytes,
  *               or NULL.  Three uses.
- *               (0) add=0 and bstride < bsize, where the kernel cannot order the blocks itself (NHWC stack,
- *               long lists, more than 2x2 blocks over a pixel): every block writes only the pixels that no
+ *               (0) add=0 and bstride < bsize, where the kernel cannot order the blocks itself (long lists,
+ *               more than 2x2 blocks over a pixel): every block writes only the pixels that no
  *               block listed later covers: the CPU functor's result, no pixel written twice.  Which pixels
  *               those are comes from one small extra launch that compares the blocks of the list pairwise (at
  *               most 2x2 blocks over a pixel and at most 4096 blocks; in-place op), or else from an owner map

@@ -6,6 +6,8 @@
 
 namespace sbnet {
 
+constexpr int NHWC_RANK_ROWS = 3;  // list rows per lane that the NHWC kernel fetches at once when it ranks its block
+
 // sparse_gather.cc:103-130 with transpose == false.
 template <int VEC, int MODE>
 __global__ __launch_bounds__(256) void k_scatter_nhwc_wide(const float* __restrict__ x, float* y, const float* ysrc,
@@ -127,11 +129,47 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
             own[u] = __builtin_bit_cast(int32_t, buf_load<1>(wr, ok ? pix * 4u : BUF_OOB));
         }
     }
-    if (MODE == SCATTER_OWNED) {
+    if (MODE == SCATTER_RANKED_INLINE) {
+        // The wave ranks its block against the rows listed after it: NHWC_RANK_ROWS rows per lane, fetched behind
+        // the wave's own loads (they are there when its data is), OR-reduced over the wave; pixels of a class that
+        // a later row covers are not stored (their loads were issued for nothing: two rows and columns of a block).
+        const uint32_t listCount = list_count(a.g, fdiv(a.units, a.dCpb));
+        const ListRows lr = list_rows(idx, listCount);
+        ListRow rows[NHWC_RANK_ROWS];
+#pragma unroll
+        for (int u = 0; u < NHWC_RANK_ROWS; ++u) {
+            const uint32_t j = ib + 1u + (uint32_t)u * 64u + lane;
+            rows[u] = list_row_load(lr, j, j < listCount);
+        }
+        uint32_t bits = 0u;
+#pragma unroll
+        for (int u = 0; u < NHWC_RANK_ROWS; ++u) {
+            int n2, bh2, bw2;
+            list_row_unpack(rows[u], n2, bh2, bw2);
+            if (ib + 1u + (uint32_t)u * 64u + lane < listCount) bits |= rank_pair_bits(o.n, o.bh, o.bw, n2, bh2, bw2);
+        }
+        for (uint32_t j = ib + 1u + (uint32_t)NHWC_RANK_ROWS * 64u + lane; j < listCount; j += 64u) {
+            int n2, bh2, bw2;
+            list_row_unpack(list_row_load(lr, j, true), n2, bh2, bw2);
+            bits |= rank_pair_bits(o.n, o.bh, o.bw, n2, bh2, bw2);
+        }
+        // most waves see none of the few neighbouring rows
+        if (__ballot(bits != 0u) != 0ull) {
+            for (int off = 32; off > 0; off >>= 1) bits |= (uint32_t)__shfl_xor((int)bits, off);
+#pragma unroll
+            for (int u = 0; u < NHWC_UNR; ++u) {
+                const uint32_t e = e0 + u * 64;
+                const uint32_t r = fdiv(e, a.dRow);
+                if (ranked_out(bits, r, fdiv(e - r * a.rowV, a.dCV), a.g)) dst[u] = BUF_OOB;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < NHWC_UNR; ++u) buf_store<BUF_NT>(yr, dst[u], v[u]);
+    } else if (MODE == SCATTER_OWNED) {
         // (an out-of-range owner read returns 0, which may equal ib: dst is BUF_OOB there already)
 #pragma unroll
         for (int u = 0; u < NHWC_UNR; ++u) buf_store<BUF_NT>(yr, own[u] == (int32_t)ib ? dst[u] : BUF_OOB, v[u]);
-    } else if (MODE == SCATTER_ASSIGN || MODE == SCATTER_RANKED || MODE == SCATTER_RANKED_INLINE) {
+    } else if (MODE == SCATTER_ASSIGN || MODE == SCATTER_RANKED) {
 #pragma unroll
         for (int u = 0; u < NHWC_UNR; ++u) buf_store<BUF_NT>(yr, dst[u], v[u]);
     } else if (MODE == SCATTER_ADD || (MODE == SCATTER_COLOR && !atomics)) {
@@ -2005,14 +2043,19 @@ static bool build_owner_map(const int16_t* idx, int numActive, const Geom& g, vo
     return true;
 }
 
-// The planar tile kernel can rank the blocks itself (SCATTER_RANKED_INLINE): planar stack, at most 2x2 blocks over
-// a pixel, a list short enough that a workgroup's share of the comparison stays small against its tile.
+// The kernels can rank the blocks themselves (SCATTER_RANKED_INLINE): at most 2x2 blocks over a pixel, a list short
+// enough that the comparison stays small against the data moved: a workgroup of the planar tile kernel compares
+// once per 16-24 KB tile, a wave of the NHWC kernel once per 4 KB, which makes that kernel about a fifth slower:
+// worth it while the launch of k_rank_table (4-5 us) costs more, up to about 200 blocks of the 800x800x128 workload.
 constexpr int RANK_INLINE_MAX_BLOCKS = 2048;
+constexpr int RANK_INLINE_MAX_BLOCKS_NHWC = 64 * NHWC_RANK_ROWS;
 
 static bool rank_inline_applies(const Geom& g, int numActive, bool transpose, int vec)
 {
-    if (!transpose || numActive > RANK_INLINE_MAX_BLOCKS || !(g.U < g.R || g.V < g.S)) return false;
+    if (numActive > RANK_INLINE_MAX_BLOCKS || !(g.U < g.R || g.V < g.S)) return false;
     if (g.R > 2 * (int64_t)g.U || g.S > 2 * (int64_t)g.V || (int64_t)g.R * g.S < 4) return false;
+    // (the wide NHWC kernel, for images beyond 32-bit offsets, does not rank)
+    if (!transpose) return numActive <= RANK_INLINE_MAX_BLOCKS_NHWC && nhwc_fits_buffers(g);
     TileArgs a;
     int threads;
     size_t lds;

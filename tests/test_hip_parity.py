@@ -756,16 +756,17 @@ def test_overlapping_plain_writes_follow_list_order(geom):
         yv = dev(base)
         sbnet_amd.sparse_scatter_var(sd, cnt, idxd, yv, bs, bst, bo, add=False, transpose=transpose)
         np.testing.assert_array_equal(host(yv), y_o)
-        if transpose and bs[0] <= 2 * bst[0] and bs[1] <= 2 * bst[1] and bs[0] * bs[1] >= 4:
-            # planar stack, at most 2x2 blocks over a pixel: the in-place op needs no scratch for the order (the
-            # kernel compares the list itself; lists longer than a workgroup's first fetch included)
+        if (transpose or M <= 192) and bs[0] <= 2 * bst[0] and bs[1] <= 2 * bst[1] and bs[0] * bs[1] >= 4:
+            # at most 2x2 blocks over a pixel (and, for an NHWC stack, at most 192 blocks): the in-place op needs no
+            # scratch for the order (the kernel compares the list itself; lists longer than a workgroup's first
+            # fetch included)
             yv = dev(base)
-            ops.scatter_forward(sd, cnt, idxd, yv, bs, bst, bo, False, False, True, use_var=True, scratch=False)
+            ops.scatter_forward(sd, cnt, idxd, yv, bs, bst, bo, False, False, transpose, use_var=True, scratch=False)
             np.testing.assert_array_equal(host(yv), y_o)
             yv = dev(base)
-            ops.scatter_forward(sd, dcount, idxd, yv, bs, bst, bo, False, False, True, use_var=True, scratch=False)
+            ops.scatter_forward(sd, dcount, idxd, yv, bs, bst, bo, False, False, transpose, use_var=True, scratch=False)
             np.testing.assert_array_equal(host(yv), orc.sparse_scatter(stack, [M - 2], idx, base, bs, bst, bo, add=False,
-                                                                        transpose=True))
+                                                                        transpose=transpose))
         # the count on the device: the last two rows of the list do not take part
         y_o2 = orc.sparse_scatter(stack, [M - 2], idx, base, bs, bst, bo, add=False, transpose=transpose)
         yv = dev(base)
