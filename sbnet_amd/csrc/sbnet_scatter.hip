@@ -1989,20 +1989,27 @@ __global__ __launch_bounds__(256) void k_rank_table(const int16_t* __restrict__ 
                                                     int32_t* __restrict__ table)
 {
     const uint32_t lane = threadIdx.x & 63u;
-    const int ib = (int)(blockIdx.x * 4u + (threadIdx.x >> 6));
-    int count = numActive;
-    if (g.countDev) count = min(count, *g.countDev);
+    const uint32_t ib = (uint32_t)__builtin_amdgcn_readfirstlane((int)(blockIdx.x * 4u + (threadIdx.x >> 6)));
+    const uint32_t count = list_count(g, (uint32_t)numActive);
     if (ib >= count) return;
-    const int n = idx[(size_t)ib * 3], bh = idx[(size_t)ib * 3 + 1], bw = idx[(size_t)ib * 3 + 2];
+    const RawTriple raw = load_triple(idx, ib);
+    const ListRows lr = list_rows(idx, count);
     uint32_t bits = 0u;
-    for (int j = ib + 1 + (int)lane; j < count; j += 64) {
-        const int dn = idx[(size_t)j * 3] - n, dh = idx[(size_t)j * 3 + 1] - bh, dw = idx[(size_t)j * 3 + 2] - bw;
-        if (dn == 0 && dh >= -1 && dh <= 1 && dw >= -1 && dw <= 1) {
-            // row classes (0: first R-U rows, 1: middle, 2: rows from U on) that a block dh steps away covers
-            const uint32_t rows = dh < 0 ? 1u : (dh > 0 ? 4u : 7u), cols = dw < 0 ? 1u : (dw > 0 ? 4u : 7u);
+    // eight rows per lane in flight (one 8-byte load each): the kernel is a chain of load latencies and nothing else
+    constexpr int UNR = 8;
+    for (uint32_t j0 = ib + 1u; j0 < count; j0 += 64u * UNR) {
+        ListRow rows[UNR];
 #pragma unroll
-            for (int rc = 0; rc < 3; ++rc)
-                if (rows & (1u << rc)) bits |= cols << (3 * rc);
+        for (int u = 0; u < UNR; ++u) {
+            const uint32_t j = j0 + (uint32_t)u * 64u + lane;
+            rows[u] = list_row_load(lr, j, j < count);
+        }
+        const BlockOrigin o = origin_of(raw, g);
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) {
+            int n2, bh2, bw2;
+            list_row_unpack(rows[u], n2, bh2, bw2);
+            if (j0 + (uint32_t)u * 64u + lane < count) bits |= rank_pair_bits(o.n, o.bh, o.bw, n2, bh2, bw2);
         }
     }
     for (int off = 32; off > 0; off >>= 1) bits |= (uint32_t)__shfl_xor((int)bits, off);
