@@ -434,6 +434,42 @@ def cpu_baseline(wl, M, idx_host, nbytes, budget_s=12.0):
              "ms_per_pass": round(tm * 1e3, 2)})
 
 
+def copy_rate(torch, lib, batches=7, reps=24):
+    """What a flat copy reaches on this box: the library's copy kernel (sbnet_copy_tensor: nontemporal 16-byte loads
+    and stores, 16 KB per workgroup) on 256 MiB, three rotating buffer pairs, timed like the ops (HIP events around
+    batches of back-to-back launches on the launch stream).  The block movers are copies with index arithmetic, so
+    this is the practical ceiling their rates are to be read against, beside the 8 TB/s of the data sheet."""
+    n = 64 * 1024 * 1024  # floats
+    src = [torch.ones(n, device="cuda:0") for _ in range(3)]
+    dst = [torch.empty(n, device="cuda:0") for _ in range(3)]
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def fn(i):
+        rc = lib.sbnet_copy_tensor(dst[i % 3].data_ptr(), src[i % 3].data_ptr(), n, st)
+        assert rc == 0
+
+    for i in range(3):
+        fn(i)
+    torch.cuda.synchronize()
+    per = []
+    for b in range(batches):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        fn(0)
+        fn(1)
+        e0.record()
+        for r in range(reps):
+            fn(b * reps + r)
+        e1.record()
+        e1.synchronize()
+        per.append(e0.elapsed_time(e1) * 1e3 / reps)
+    us = statistics.median(per)
+    del src, dst
+    torch.cuda.empty_cache()
+    gbps = 2 * n * 4 / us * 1e-3
+    return {"kernel": "k_copy_v4 (sbnet_copy_tensor), 256 MiB read + 256 MiB written per launch", "us": round(us, 2),
+            "GBps": round(gbps, 1), "frac_of_8TBps": round(gbps / HBM_PEAK_GBS, 4)}
+
+
 def kernel_source_digest():
     """sha256 over the code of the device sources the library is built from (csrc/*.hip and csrc/*.h, by name,
     comments and white space left out): the counters under profiles/ belong to one state of it."""
@@ -620,6 +656,10 @@ def main():
     if traffic:
         # the same launch time against the bytes the profiler counted between L2 and the fabric
         roofline["traffic_GBps"] = round(traffic / g["us"] * 1e-3, 1)
+    # a flat copy on the same box, timed the same way: what a copy-shaped kernel can reach here
+    flat = copy_rate(torch, lib)
+    roofline["flat_copy"] = flat
+    roofline["frac_of_flat_copy"] = round(g["GBps"] / flat["GBps"], 4)
     out = {
         "metric": "achieved HBM GB/s over reduce_mask+sparse_gather+sparse_scatter_var (algorithmic bytes / wall time per step); us/op and % of HBM peak under ops, ops_by_density and roofline",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
