@@ -6,7 +6,7 @@
 
 namespace sbnet {
 
-constexpr int NHWC_RANK_ROWS = 3;  // list rows per lane that the NHWC kernel fetches at once when it ranks its block
+constexpr int NHWC_RANK_ROWS = 1;  // list rows per thread that the NHWC kernel fetches at once when it ranks its block
 
 // sparse_gather.cc:103-130 with transpose == false.
 template <int VEC, int MODE>
@@ -112,6 +112,31 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
     if (MODE == SCATTER_SUM && !repeats) nb = neighbour_positions(col, o, ib);
     const rsrc_t wr = make_rsrc(MODE == SCATTER_OWNED ? col.owner + (int64_t)o.n * a.g.H * a.g.W : nullptr,
                                 MODE == SCATTER_OWNED ? (uint32_t)(a.g.H * a.g.W) * 4u : 0u);
+    // SCATTER_RANKED_INLINE: the block is ranked against the rows listed after it inside the kernel.  The rows are
+    // fetched AHEAD of the wave's own loads, so they arrive first and are compared while the data is still on its
+    // way (loads return in order): the stores wait no longer than they would anyway.  The four waves of a workgroup
+    // mostly move the same block: they then share the comparison, NHWC_RANK_ROWS rows per thread, and meet at one
+    // barrier; a workgroup whose waves move two blocks compares per wave.
+    __shared__ uint32_t waveBits[4];
+    ListRow rows[NHWC_RANK_ROWS];
+    ListRows lr;
+    uint32_t listCount = 0, me = lane, step = 64u;
+    const uint32_t unit0 = blockIdx.x * 4u;
+    bool shared = false;
+    if (MODE == SCATTER_RANKED_INLINE) {
+        listCount = list_count(a.g, fdiv(a.units, a.dCpb));
+        lr = list_rows(idx, listCount);
+        shared = fdiv(unit0, a.dCpb) == fdiv(min(unit0 + 3u, a.units - 1u), a.dCpb);  // (the same for the whole workgroup)
+        if (shared) {
+            me = threadIdx.x;
+            step = 256u;
+        }
+#pragma unroll
+        for (int u = 0; u < NHWC_RANK_ROWS; ++u) {
+            const uint32_t j = ib + 1u + (uint32_t)u * step + me;
+            rows[u] = list_row_load(lr, j, j < listCount);
+        }
+    }
 #pragma unroll
     for (int u = 0; u < NHWC_UNR; ++u) {
         const uint32_t e = e0 + u * 64;
@@ -130,32 +155,33 @@ __global__ __launch_bounds__(256) void k_scatter_nhwc(const float* __restrict__ 
         }
     }
     if (MODE == SCATTER_RANKED_INLINE) {
-        // The wave ranks its block against the rows listed after it: NHWC_RANK_ROWS rows per lane, fetched behind
-        // the wave's own loads (they are there when its data is), OR-reduced over the wave; pixels of a class that
-        // a later row covers are not stored (their loads were issued for nothing: two rows and columns of a block).
-        const uint32_t listCount = list_count(a.g, fdiv(a.units, a.dCpb));
-        const ListRows lr = list_rows(idx, listCount);
-        ListRow rows[NHWC_RANK_ROWS];
-#pragma unroll
-        for (int u = 0; u < NHWC_RANK_ROWS; ++u) {
-            const uint32_t j = ib + 1u + (uint32_t)u * 64u + lane;
-            rows[u] = list_row_load(lr, j, j < listCount);
-        }
+        // pixels of a class that a later row covers are not stored (their loads were issued for nothing: two rows
+        // and columns of a block)
         uint32_t bits = 0u;
 #pragma unroll
         for (int u = 0; u < NHWC_RANK_ROWS; ++u) {
             int n2, bh2, bw2;
             list_row_unpack(rows[u], n2, bh2, bw2);
-            if (ib + 1u + (uint32_t)u * 64u + lane < listCount) bits |= rank_pair_bits(o.n, o.bh, o.bw, n2, bh2, bw2);
+            if (ib + 1u + (uint32_t)u * step + me < listCount) bits |= rank_pair_bits(o.n, o.bh, o.bw, n2, bh2, bw2);
         }
-        for (uint32_t j = ib + 1u + (uint32_t)NHWC_RANK_ROWS * 64u + lane; j < listCount; j += 64u) {
+        for (uint32_t j = ib + 1u + (uint32_t)NHWC_RANK_ROWS * step + me; j < listCount; j += step) {
             int n2, bh2, bw2;
             list_row_unpack(list_row_load(lr, j, true), n2, bh2, bw2);
             bits |= rank_pair_bits(o.n, o.bh, o.bw, n2, bh2, bw2);
         }
         // most waves see none of the few neighbouring rows
-        if (__ballot(bits != 0u) != 0ull) {
+        if (__ballot(bits != 0u) != 0ull)
             for (int off = 32; off > 0; off >>= 1) bits |= (uint32_t)__shfl_xor((int)bits, off);
+        if (shared) {
+            if (lane == 0u) waveBits[threadIdx.x >> 6] = bits;
+            lds_barrier();
+            // (waves past the last unit have left before the barrier, which waits for the surviving ones only)
+            bits = 0u;
+#pragma unroll
+            for (uint32_t w = 0; w < 4u; ++w)
+                if (unit0 + w < a.units) bits |= waveBits[w];
+        }
+        if (bits != 0u) {
 #pragma unroll
             for (int u = 0; u < NHWC_UNR; ++u) {
                 const uint32_t e = e0 + u * 64;
@@ -2052,10 +2078,11 @@ static bool build_owner_map(const int16_t* idx, int numActive, const Geom& g, vo
 
 // The kernels can rank the blocks themselves (SCATTER_RANKED_INLINE): at most 2x2 blocks over a pixel, a list short
 // enough that the comparison stays small against the data moved: a workgroup of the planar tile kernel compares
-// once per 16-24 KB tile, a wave of the NHWC kernel once per 4 KB, which makes that kernel about a fifth slower:
-// worth it while the launch of k_rank_table (4-5 us) costs more, up to about 200 blocks of the 800x800x128 workload.
+// once per 16-24 KB tile; a wave of the NHWC kernel moves 4 KB and is slowed by every instruction on its way (with 312
+// blocks that kernel takes 39 us against 34), which is worth it while the launch of k_rank_table (3-5 us) costs
+// more: up to about 200 blocks of the 800x800x128 workload.
 constexpr int RANK_INLINE_MAX_BLOCKS = 2048;
-constexpr int RANK_INLINE_MAX_BLOCKS_NHWC = 64 * NHWC_RANK_ROWS;
+constexpr int RANK_INLINE_MAX_BLOCKS_NHWC = 192;
 
 static bool rank_inline_applies(const Geom& g, int numActive, bool transpose, int vec)
 {
