@@ -4,6 +4,8 @@ import os
 import subprocess
 import sys
 
+import pytest
+
 import bench
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -67,3 +69,48 @@ def test_bench_structs_match_the_cxx_loop():
     lib.sbnet_bench_struct_bytes.restype = ctypes.c_size_t
     assert lib.sbnet_bench_struct_bytes(0) == ctypes.sizeof(bench.BenchSet) == 96
     assert lib.sbnet_bench_struct_bytes(1) == ctypes.sizeof(bench.BenchGeom)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["config1", "config2", "config4_small"])
+def test_cxx_host_loop_matches_the_oracle(name):
+    """The C++ host loop that bench.py times (libsbnet_bench.so) runs the same step as the Python mirror: with a mask
+    and a gather (copying scatter at the end), and with a given block list and no gather (in-place atomic add).  Its
+    outputs are compared with the CPU oracle, so that the timed step is known to be the op sequence it claims."""
+    import numpy as np
+    import torch
+    from oracle import sbnet_oracle as orc
+    from sbnet_amd import _lib, workloads
+    lib = _lib.load()
+    torch.cuda.set_device(0)
+    if name == "config4_small":
+        # the overlapping scatter-add configuration's geometry on a small base, block list given
+        rng = np.random.default_rng(7)
+        cells = np.array([(n, i, j) for n in range(2) for i in range(8) for j in range(8) if rng.random() < 0.3], np.int16)
+        wl = workloads.config4()._replace(shape=[2, 64, 64, 32], bcount=[8, 8], indices=cells, name="C4-small")
+    else:
+        wl = getattr(workloads, name)()
+    p = bench.Path(wl, torch, lib, nsets=2)
+    if wl.x is None:
+        for s in p.sets:
+            s["base"].zero_()
+    before = [s["base"].clone() for s in p.sets]
+    ms = bench.cxx_pipeline(p, 2, 0, 1, device_count=False)["host_count"]   # two steps per call: each set once
+    assert ms > 0
+    torch.cuda.synchronize()
+    M = p.M
+    idx = p.idx_host[:M]
+    cnt = np.array([M], np.int32)
+    for k, s in enumerate(p.sets):
+        stack = s["sstack"].cpu().numpy()[:M]
+        if wl.x is not None and s["sstack"] is s["stack"]:
+            # the loop gathers into a stack of its own (the list's capacity): take the oracle's gather instead
+            stack = orc.sparse_gather(wl.x, cnt, idx, wl.bsize, wl.bstride, wl.boffset, transpose=wl.transpose)
+        base0 = before[k].cpu().numpy()
+        calls = 2 if wl.s_var else 1   # (the loop ran warm-up + timed batch: the in-place op has been applied twice)
+        exp = base0
+        for _ in range(calls):
+            exp = orc.sparse_scatter(stack, cnt, idx, exp, wl.s_bsize, wl.s_bstride, wl.s_boffset, add=wl.s_add,
+                                     atomic=wl.s_atomic, transpose=wl.transpose)
+        got = (s["base"] if wl.s_var else s["out"]).cpu().numpy()
+        np.testing.assert_array_equal(got, exp)
