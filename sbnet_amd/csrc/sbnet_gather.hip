@@ -168,7 +168,7 @@ __global__ __launch_bounds__(512) void k_gather_planar(const float* __restrict__
 }
 
 // ---------------------------------------------------------------------------------------------
-// Planar gather whose workgroups own whole 128-byte lines of the output
+// Planar gather whose workgroups own whole, aligned 64-byte pieces ("lines") of the output
 // ---------------------------------------------------------------------------------------------
 //
 // A write-only probe of the tile pattern above (32 runs of 243 floats at 729-float pitch, 4-byte
@@ -180,12 +180,16 @@ __global__ __launch_bounds__(512) void k_gather_planar(const float* __restrict__
 // [c*RS + p0, c*RS + p1): the range [up(c*RS + p0), up(c*RS + p1)), up() rounding to the next line of
 // y (the two ends of the chunk stay where they are).  These ranges tile the chunk exactly, every store
 // is an aligned dwordx4, and no line is written by two workgroups (except the one line two chunks may
-// share).  The price is that a tile needs up to 31 pixels beyond p1 -- for the last split of a plane,
-// where row c's last line runs into row c+1, the first 31 pixels of the plane -- so the tile's pixel
-// window is [p0, p1 + LINE_EXT) taken cyclically over the plane, about 13 % more NHWC reads at 243
-// pixels per tile; the extra pixels are read by the neighbouring tile as well and come from cache (a
-// bare read-and-write of this access pattern takes the same time with and without them).  Used when a
-// plane is split over several tiles; a tile of whole planes already writes one contiguous piece.
+// share).  The price is that a tile needs up to LINE_EXT pixels beyond p1 -- for the last split of a
+// plane, where row c's last line runs into row c+1, the first pixels of the plane -- so the tile's pixel
+// window is [p0, p1 + LINE_EXT) taken cyclically over the plane; the extra pixels are read by the
+// neighbouring tile as well and mostly come from cache.  Used when a plane is split over several tiles;
+// a tile of whole planes already writes one contiguous piece.
+//
+// The unit of ownership is 64 bytes, the granularity of an access to HBM, not the 128 bytes of an L2 line: with
+// 16-float units a tile reads 15 extra pixels instead of 31 (6 % instead of 13 % more NHWC reads at 243 pixels
+// per tile) and the launch on 312 blocks of 27x27x128 takes 39.05 us instead of 39.6; 32-byte units are no
+// faster than 128-byte ones (39.5 us, and 8.8 against 7.5 us on 58 blocks).
 //
 // LDS: row c at c*Pp, window pixel q at column q + phi(c), phi(c) = (c*RS + p0) & 3, XOR-swizzled as
 // above.  The shift phi makes LDS columns congruent to l modulo 4, so every output slot is one
@@ -193,7 +197,7 @@ __global__ __launch_bounds__(512) void k_gather_planar(const float* __restrict__
 // stored behind the pixels of channel c-1 instead, where l continues: the slots of row c-1's last line
 // that cross into plane c are then contiguous in LDS like any other.
 
-constexpr int LINE_FLOATS = 32;
+constexpr int LINE_FLOATS = 16;
 constexpr int LINE_EXT = LINE_FLOATS - 1;
 
 struct LineArgs {

@@ -57,6 +57,9 @@ def test_tiles_fit_the_kernels(kind):
     assert short_tails > 0
 
 
+LINE = 16  # floats per unit of ownership of the line-owning gather: 64 bytes
+
+
 def test_line_owning_gather_tiles():
     used = 0
     for R, S in itertools.product(SIZES, [5, 16, 18, 27, 31, 63, 65]):
@@ -70,8 +73,8 @@ def test_line_owning_gather_tiles():
                     used += 1
                     tag = (R, S, C, num_active, align, t)
                     assert t["psplit"] >= 2 and (t["psplit"] - 1) * t["P"] < RS <= t["psplit"] * t["P"], tag
-                    assert t["last"] >= 32, tag                       # the last split holds the 31-pixel extension
-                    assert t["Pp"] % 32 == 0 and t["Pp"] >= t["P"] + 31 + 3, tag
+                    assert t["last"] >= LINE, tag                     # the last split holds the extension
+                    assert t["Pp"] % 32 == 0 and t["Pp"] >= t["P"] + LINE - 1 + 3, tag
                     assert t["lds"] == t["Ct"] * t["Pp"] * 4 <= 64 * 1024, tag
                     assert 4 <= t["have"] <= 8 and t["need"] <= t["have"], tag
     assert used > 100
