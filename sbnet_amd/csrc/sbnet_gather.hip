@@ -500,8 +500,8 @@ static bool make_line_args(const Geom& g, int numActive, const float* y, LineArg
     return true;
 }
 
-// 5 vectors per thread (three splits of a 27x27 plane) for launches of many workgroups, 7 (two splits: fewer
-// window pixels read twice, more bytes in flight per workgroup) for launches of few, as for the scatter:
+// 5 vectors per thread (three splits of a 27x27 plane) for launches of many workgroups, up to 7 (two splits, which
+// take 6: fewer window pixels read twice, more bytes in flight per workgroup) for launches of few, as for the scatter:
 // 8.62 -> 7.76 us at 58 blocks, 21.7 -> 20.8 us at 156, but 31.1 -> 31.6 us at 231 and 40.3 -> 40.6 us at 312.
 constexpr int GATHER_FEW_WGS_PER_CU = 9;
 
