@@ -247,8 +247,8 @@ size_t sbnet_sparse_scatter_workspace_bytes(int32_t num_active, const int64_t* y
  *               most 2x2 blocks over a pixel and at most 4096 blocks; in-place op), or else from an owner map
  *               (one int32 per pixel: the last listed block that covers it) built by two extra launches.
  *               (1) sbnet_sparse_scatter with atomic=0 and blocks that do not overlap (bstride >= bsize): y is
- *               built in one pass over its bytes instead of "copy ybase, scatter on top".  Two small launches
- *               put an inverse map (block position -> list position) into the scratch; one streaming kernel
+ *               built in one pass over its bytes instead of "copy ybase, scatter on top".  One or two small
+ *               launches put an inverse map (block position -> list position) into the scratch; one streaming kernel
  *               then walks y in row order, reads ybase where the result needs it (all of it for an add, the
  *               uncovered pixels for a plain write), reads the block stack where a block covers the pixel and
  *               writes y once.  Same y, every byte moved once.  A list that names a block several times gets
@@ -256,10 +256,13 @@ size_t sbnet_sparse_scatter_workspace_bytes(int32_t num_active, const int64_t* y
  *               all of them in list order).  A planar stack (transpose=1) is staged through LDS by the same
  *               kernel when bsize[1] and bstride[1] are multiples of 4, bstride[1] divides the kernel's strip
  *               width (256 channel vectors, i.e. 32 pixels at 32 channels or more) and boffset[1] is a
- *               multiple of bstride[1]; other planar geometries take two passes once the blocks cover 16 MB
- *               (copy of the uncovered pixels, then the scatter kernel, which reads ybase where it adds), and
- *               copy-then-scatter below that: in these two cases rows that name the same block race as they
- *               do in the reference's GPU kernels.  Overlapping plain writes (add=0, bstride < bsize) from
+ *               multiple of bstride[1]; other planar geometries whose blocks tile the plane (bsize == bstride,
+ *               cells of 4 KB or more) are built by one launch over the cells of the block grid (a cell with a
+ *               block from the stack, an empty cell from ybase; exact for repeated rows as well); the remaining
+ *               planar geometries take two passes once the blocks cover 16 MB (copy of the uncovered pixels,
+ *               then the scatter kernel, which reads ybase where it adds), and copy-then-scatter below that:
+ *               in these two cases rows that name the same block race as they do in the reference's GPU
+ *               kernels.  Overlapping plain writes (add=0, bstride < bsize) from
  *               16 MB of blocks on use the owner map of (0) as their coverage record in the same way.
  *               (2) add=1, atomic=1: with it the overlapping adds need no atomics:
  *               - transpose=0 and at most 2x2 blocks per pixel: each pixel is summed by one owner in ascending
