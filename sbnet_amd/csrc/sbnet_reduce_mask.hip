@@ -78,7 +78,7 @@ __device__ __forceinline__ float next_down(float f)
 
 __device__ __forceinline__ float next_up(float f) { return -next_down(-f); }
 
-constexpr int POOL_LD = 8;  // loads in flight per lane
+constexpr int POOL_LD = 12;  // loads in flight per lane (a 6x6 window over 4 lanes is 9 loads each: one round, not 8 + 1)
 
 __global__ __launch_bounds__(256) void k_reduce_pool(const float* __restrict__ mask, PoolArgs a,
                                                      uint8_t* __restrict__ flags, int32_t* __restrict__ counts)
